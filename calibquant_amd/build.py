@@ -1,0 +1,64 @@
+"""Build the C-ABI HIP library in-tree: calibquant_amd/lib/libcalibquant_hip.so.
+
+Run `python -m calibquant_amd.build`.  hipcc cross-compiles for gfx950 without
+a GPU.  The built library is git-ignored and is loaded by `calibquant_amd._lib`.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+LIBDIR = os.path.join(HERE, "lib")
+LIBPATH = os.path.join(LIBDIR, "libcalibquant_hip.so")
+SOURCES = ["cq_core.hip", "cq_quantize.hip", "cq_lutvecmat.hip", "cq_decode.hip"]
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC",
+    "-fhip-fp32-correctly-rounded-divide-sqrt",
+    # keep the compiler from emitting packed-fp32 VALU ops
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-command-line-argument",
+    "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
+]
+
+
+def build(verbose: bool = True, jobs: int = 4) -> str:
+    os.makedirs(LIBDIR, exist_ok=True)
+    objs, procs = [], []
+    for src in SOURCES:
+        obj = os.path.join(LIBDIR, src.replace(".hip", ".o"))
+        objs.append(obj)
+        cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        if len(procs) >= jobs:
+            _drain(procs)
+    _drain(procs)
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIBPATH, *objs]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    return LIBPATH
+
+
+def _drain(procs):
+    while procs:
+        src, p = procs.pop(0)
+        out, _ = p.communicate()
+        # hipcc's host pass warns that it does not know the packed-fp32 feature; harmless
+        out = "\n".join(l for l in out.splitlines() if "packed-fp32-ops" not in l)
+        if out.strip():
+            print(out)
+        if p.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {src}")
+
+
+if __name__ == "__main__":
+    print(build())
+    sys.exit(0)

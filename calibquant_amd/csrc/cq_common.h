@@ -1,0 +1,113 @@
+// Shared device helpers for the gfx950 CalibQuant kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include "calibquant_hip.h"
+
+namespace cq {
+
+constexpr int kWave = 64;
+
+// Last HIP runtime error seen by this host thread (cq_last_hip_error()).
+extern thread_local int g_last_hip_error;
+
+inline int hip_fail(hipError_t e) {
+    g_last_hip_error = static_cast<int>(e);
+    return CQ_ERR_LAUNCH;
+}
+
+#define CQ_HIP_CHECK(expr)                                 \
+    do {                                                   \
+        hipError_t _e = (expr);                            \
+        if (_e != hipSuccess) return ::cq::hip_fail(_e);   \
+    } while (0)
+
+#define CQ_LAUNCH_CHECK()                                  \
+    do {                                                   \
+        hipError_t _e = hipGetLastError();                 \
+        if (_e != hipSuccess) return ::cq::hip_fail(_e);   \
+    } while (0)
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---------------------------------------------------------------- dtypes
+struct BF16 {};
+struct FP16 {};
+
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t h) { return __uint_as_float(h << 16); }
+
+// fp32 -> bf16 bits, round to nearest even, NaN kept quiet.
+__device__ __forceinline__ uint32_t float_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+
+__device__ __forceinline__ float fp16_bits_to_float(uint32_t h) {
+    return __half2float(__ushort_as_half(static_cast<unsigned short>(h)));
+}
+
+__device__ __forceinline__ uint32_t float_to_fp16_bits(float f) {
+    return static_cast<uint32_t>(__half_as_ushort(__float2half_rn(f)));
+}
+
+template <typename DT> struct Cvt;
+template <> struct Cvt<BF16> {
+    static __device__ __forceinline__ float to_float(uint32_t bits16) { return bf16_bits_to_float(bits16); }
+    static __device__ __forceinline__ uint32_t from_float(float f) { return float_to_bf16_bits(f); }
+    // low / high halves of a 32-bit word holding two elements
+    static __device__ __forceinline__ float lo(uint32_t w) { return __uint_as_float(w << 16); }
+    static __device__ __forceinline__ float hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+};
+template <> struct Cvt<FP16> {
+    static __device__ __forceinline__ float to_float(uint32_t bits16) { return fp16_bits_to_float(bits16); }
+    static __device__ __forceinline__ uint32_t from_float(float f) { return float_to_fp16_bits(f); }
+    static __device__ __forceinline__ float lo(uint32_t w) { return fp16_bits_to_float(w & 0xffffu); }
+    static __device__ __forceinline__ float hi(uint32_t w) { return fp16_bits_to_float(w >> 16); }
+};
+
+// Round an fp32 value to the storage dtype and back (one torch op boundary).
+template <typename DT>
+__device__ __forceinline__ float rnd(float f) { return Cvt<DT>::to_float(Cvt<DT>::from_float(f)); }
+
+// 8 consecutive 16-bit elements (one 16-byte load) -> 8 floats
+template <typename DT>
+__device__ __forceinline__ void unpack8(const uint4& v, float* f) {
+    f[0] = Cvt<DT>::lo(v.x); f[1] = Cvt<DT>::hi(v.x);
+    f[2] = Cvt<DT>::lo(v.y); f[3] = Cvt<DT>::hi(v.y);
+    f[4] = Cvt<DT>::lo(v.z); f[5] = Cvt<DT>::hi(v.z);
+    f[6] = Cvt<DT>::lo(v.w); f[7] = Cvt<DT>::hi(v.w);
+}
+
+template <typename DT>
+__device__ __forceinline__ float load_elem(const void* p, int64_t i) {
+    return Cvt<DT>::to_float(static_cast<const uint16_t*>(p)[i]);
+}
+
+template <typename DT>
+__device__ __forceinline__ void store_elem(void* p, int64_t i, float f) {
+    static_cast<uint16_t*>(p)[i] = static_cast<uint16_t>(Cvt<DT>::from_float(f));
+}
+
+// ------------------------------------------------------- wave reductions
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+    return v;
+}
+__device__ __forceinline__ float wave_min(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, kWave));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+
+}  // namespace cq

@@ -1,0 +1,319 @@
+// Prefill quantise-and-pack for gfx950, and the unfused quant()/encode()
+// operators of the reference surface.
+//
+// Per-channel statistics need a column reduction over the token axis, so the
+// work is three launches on one stream:
+//   1. partial min/max per (batch, head, token chunk, channel)  - reads x once
+//   2. statistics: combine the chunks, run the storage-dtype op chain
+//   3. emit: re-read x (L2 / Infinity Cache resident at prefill sizes),
+//      produce the codes and pack them
+// Every arithmetic step that the reference performs as a separate torch op on
+// a 16-bit tensor is rounded to that dtype here (rnd<DT>), and divisions are
+// IEEE (__fdiv_rn); contraction is off so no multiply-add is fused.
+#include "cq_common.h"
+
+#pragma clang fp contract(off)
+
+namespace cq {
+
+constexpr int kQThreads = 256;
+
+struct QuantGeom {
+    int B, T, H, D;
+    int64_t sb, st, sh;   // element strides of x
+    int nchunk, chunk;    // token chunks
+};
+
+static inline int pick_chunks(int B, int T, int H) {
+    int64_t bh = static_cast<int64_t>(B) * H;
+    int64_t want = (4096 + bh - 1) / bh;
+    int64_t cap = T / 64 > 1 ? T / 64 : 1;
+    int64_t n = want < cap ? want : cap;
+    if (n > 256) n = 256;
+    if (n < 1) n = 1;
+    return static_cast<int>(n);
+}
+
+// ---- 1. partial min / max -------------------------------------------------
+// grid (nchunk, H, B), 256 threads.  A row of D elements is covered by D/8
+// adjacent lanes with one 16-byte load each; 256/(D/8) rows per iteration.
+template <typename DT>
+__global__ __launch_bounds__(kQThreads) void minmax_partial_kernel(const uint16_t* __restrict__ x, QuantGeom g,
+                                                                  float* __restrict__ part) {
+    const int lpr = g.D >> 3;
+    const int rows_per_iter = kQThreads / lpr;
+    const int lane = threadIdx.x % lpr;
+    const int row = threadIdx.x / lpr;
+    const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int t0 = c * g.chunk;
+    const int t1 = min(g.T, t0 + g.chunk);
+    const uint16_t* base = x + b * g.sb + h * g.sh + lane * 8;
+
+    float mn[8], mx[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { mn[i] = INFINITY; mx[i] = -INFINITY; }
+    for (int t = t0 + row; t < t1; t += rows_per_iter) {
+        uint4 v = *reinterpret_cast<const uint4*>(base + t * g.st);
+        float f[8];
+        unpack8<DT>(v, f);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { mn[i] = fminf(mn[i], f[i]); mx[i] = fmaxf(mx[i], f[i]); }
+    }
+    __shared__ float smn[kQThreads * 8];
+    __shared__ float smx[kQThreads * 8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        smn[(row * lpr + lane) * 8 + i] = mn[i];
+        smx[(row * lpr + lane) * 8 + i] = mx[i];
+    }
+    __syncthreads();
+    // thread d (< D) folds the rows_per_iter partial rows of channel d
+    for (int d = threadIdx.x; d < g.D; d += kQThreads) {
+        float a = INFINITY, z = -INFINITY;
+        for (int r = 0; r < rows_per_iter; ++r) {
+            a = fminf(a, smn[r * g.D + d]);
+            z = fmaxf(z, smx[r * g.D + d]);
+        }
+        float* o = part + ((static_cast<int64_t>(b) * g.H + h) * g.nchunk + c) * 2 * g.D;
+        o[d] = a;
+        o[g.D + d] = z;
+    }
+}
+
+// ---- 2. statistics ---------------------------------------------------------
+// grid (B*H), D threads.  The op chain of calibquant.py:27-34 with one
+// rounding per op; `tensor / python_scalar` is a multiply by the fp32
+// reciprocal, as torch's device kernel does.
+template <typename DT>
+__global__ void stats_kernel(const float* __restrict__ part, QuantGeom g, float clip, float levels,
+                             uint16_t* __restrict__ scale, uint16_t* __restrict__ zero) {
+    const int bh = blockIdx.x;
+    const int d = threadIdx.x;
+    if (d >= g.D) return;
+    float a = INFINITY, z = -INFINITY;
+    const float* p = part + static_cast<int64_t>(bh) * g.nchunk * 2 * g.D;
+    for (int c = 0; c < g.nchunk; ++c) {
+        a = fminf(a, p[c * 2 * g.D + d]);
+        z = fmaxf(z, p[c * 2 * g.D + g.D + d]);
+    }
+    const float x_min = rnd<DT>(a * clip);
+    const float x_max = rnd<DT>(z * clip);
+    const float diff = rnd<DT>(x_max - x_min);
+    const float inv_levels = __fdiv_rn(1.0f, levels);
+    const float s = rnd<DT>(diff * inv_levels);
+    const float zp = rnd<DT>(__fdiv_rn(-x_min, s));
+    scale[static_cast<int64_t>(bh) * g.D + d] = static_cast<uint16_t>(Cvt<DT>::from_float(s));
+    zero[static_cast<int64_t>(bh) * g.D + d] = static_cast<uint16_t>(Cvt<DT>::from_float(zp));
+}
+
+// One element of calibquant.py:36: round(clamp(x / scale + zero_point, 0, L)).
+// Returns the rounded value; NaN stays NaN (the reference's LUT search then
+// finds no match and yields index 0).
+template <typename DT>
+__device__ __forceinline__ float quant_value(float x, float s, float zp, float levels) {
+    float y = rnd<DT>(__fdiv_rn(x, s));
+    y = rnd<DT>(y + zp);
+    if (y != y) return y;
+    y = fminf(fmaxf(y, 0.0f), levels);
+    return rintf(y);
+}
+
+// ---- 3. emit -----------------------------------------------------------------
+// XQ = false: packed codes (B, H, T, D*BITS/8).  XQ = true: the unpacked code
+// values as storage-dtype numbers in a contiguous (B, T, H, D) tensor.
+template <typename DT, int BITS, bool XQ>
+__global__ __launch_bounds__(kQThreads) void emit_kernel(const uint16_t* __restrict__ x, QuantGeom g,
+                                                        const uint16_t* __restrict__ scale,
+                                                        const uint16_t* __restrict__ zero,
+                                                        uint8_t* __restrict__ codes, uint16_t* __restrict__ xq) {
+    const int lpr = g.D >> 3;
+    const int rows_per_iter = kQThreads / lpr;
+    const int lane = threadIdx.x % lpr;
+    const int row = threadIdx.x / lpr;
+    const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int t0 = c * g.chunk;
+    const int t1 = min(g.T, t0 + g.chunk);
+    const uint16_t* base = x + b * g.sb + h * g.sh + lane * 8;
+    const int64_t bh = static_cast<int64_t>(b) * g.H + h;
+    constexpr float levels = static_cast<float>((1 << BITS) - 1);
+
+    float s[8], zp[8];
+    {
+        uint4 sv = *reinterpret_cast<const uint4*>(scale + bh * g.D + lane * 8);
+        uint4 zv = *reinterpret_cast<const uint4*>(zero + bh * g.D + lane * 8);
+        unpack8<DT>(sv, s);
+        unpack8<DT>(zv, zp);
+    }
+    const int nb = g.D * BITS / 8;  // bytes per packed row
+    for (int t = t0 + row; t < t1; t += rows_per_iter) {
+        uint4 v = *reinterpret_cast<const uint4*>(base + t * g.st);
+        float f[8];
+        unpack8<DT>(v, f);
+        float qv[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) qv[i] = quant_value<DT>(f[i], s[i], zp[i], levels);
+        if constexpr (XQ) {
+            uint32_t w[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                w[i] = Cvt<DT>::from_float(qv[2 * i]) | (Cvt<DT>::from_float(qv[2 * i + 1]) << 16);
+            uint16_t* o = xq + ((static_cast<int64_t>(b) * g.T + t) * g.H + h) * g.D + lane * 8;
+            *reinterpret_cast<uint4*>(o) = make_uint4(w[0], w[1], w[2], w[3]);
+        } else {
+            uint32_t code[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) code[i] = (qv[i] != qv[i]) ? 0u : static_cast<uint32_t>(qv[i]);
+            uint8_t* o = codes + (bh * g.T + t) * nb;
+            if constexpr (BITS == 1) {
+                uint32_t byte = 0;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) byte |= code[i] << (7 - i);
+                o[lane] = static_cast<uint8_t>(byte);
+            } else {
+                uint32_t b0 = (code[0] << 6) | (code[1] << 4) | (code[2] << 2) | code[3];
+                uint32_t b1 = (code[4] << 6) | (code[5] << 4) | (code[6] << 2) | code[7];
+                reinterpret_cast<uint16_t*>(o)[lane] = static_cast<uint16_t>(b0 | (b1 << 8));
+            }
+        }
+    }
+}
+
+template <typename DT>
+static int run_quant(const void* x, QuantGeom g, int bits, float clip, uint8_t* codes, void* xq, void* scale,
+                     void* zero, float* ws, hipStream_t st) {
+    dim3 grid(g.nchunk, g.H, g.B);
+    const uint16_t* xp = static_cast<const uint16_t*>(x);
+    uint16_t* sp = static_cast<uint16_t*>(scale);
+    uint16_t* zp = static_cast<uint16_t*>(zero);
+    hipLaunchKernelGGL(minmax_partial_kernel<DT>, grid, dim3(kQThreads), 0, st, xp, g, ws);
+    CQ_LAUNCH_CHECK();
+    const float levels = static_cast<float>((1 << bits) - 1);
+    hipLaunchKernelGGL(stats_kernel<DT>, dim3(g.B * g.H), dim3(g.D), 0, st, ws, g, clip, levels, sp, zp);
+    CQ_LAUNCH_CHECK();
+    uint16_t* xqp = static_cast<uint16_t*>(xq);
+    if (xq) {
+        if (bits == 1)
+            hipLaunchKernelGGL((emit_kernel<DT, 1, true>), grid, dim3(kQThreads), 0, st, xp, g, sp, zp, codes, xqp);
+        else
+            hipLaunchKernelGGL((emit_kernel<DT, 2, true>), grid, dim3(kQThreads), 0, st, xp, g, sp, zp, codes, xqp);
+    } else {
+        if (bits == 1)
+            hipLaunchKernelGGL((emit_kernel<DT, 1, false>), grid, dim3(kQThreads), 0, st, xp, g, sp, zp, codes, xqp);
+        else
+            hipLaunchKernelGGL((emit_kernel<DT, 2, false>), grid, dim3(kQThreads), 0, st, xp, g, sp, zp, codes, xqp);
+    }
+    CQ_LAUNCH_CHECK();
+    return CQ_OK;
+}
+
+static int quant_entry(const void* x, int dtype, int B, int T, int H, int D, int64_t sb, int64_t st, int64_t sh,
+                       int bits, float clip, uint8_t* codes, void* xq, void* scale, void* zero, void* ws,
+                       size_t ws_bytes, cq_stream_t stream) {
+    if (!x || !scale || !zero || (!codes && !xq)) return CQ_ERR_NULL;
+    if (dtype != CQ_BF16 && dtype != CQ_FP16) return CQ_ERR_DTYPE;
+    if (bits != 1 && bits != 2) return CQ_ERR_UNSUPPORTED;
+    if (B < 1 || T < 1 || H < 1 || (D != 64 && D != 128 && D != 256)) return CQ_ERR_SHAPE;
+    if (H > 65535 || B > 65535) return CQ_ERR_SHAPE;
+    if ((sb % 8) || (st % 8) || (sh % 8) || !aligned16(x) || !aligned16(scale) || !aligned16(zero) ||
+        (xq && !aligned16(xq)) || (codes && (reinterpret_cast<uintptr_t>(codes) & 1u)))
+        return CQ_ERR_ALIGN;
+    const size_t need = cq_quantize_pack_workspace(B, T, H, D);
+    if (!ws || ws_bytes < need || !aligned16(ws)) return CQ_ERR_WORKSPACE;
+    QuantGeom g;
+    g.B = B; g.T = T; g.H = H; g.D = D;
+    g.sb = sb; g.st = st; g.sh = sh;
+    g.nchunk = pick_chunks(B, T, H);
+    g.chunk = (T + g.nchunk - 1) / g.nchunk;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == CQ_BF16)
+        return run_quant<BF16>(x, g, bits, clip, codes, xq, scale, zero, static_cast<float*>(ws), s);
+    return run_quant<FP16>(x, g, bits, clip, codes, xq, scale, zero, static_cast<float*>(ws), s);
+}
+
+// ---- encode() ---------------------------------------------------------------------
+template <typename IT>
+__device__ __forceinline__ uint32_t index_of(const IT* p, int64_t i);
+template <> __device__ __forceinline__ uint32_t index_of<int64_t>(const int64_t* p, int64_t i) { return static_cast<uint32_t>(p[i]); }
+template <> __device__ __forceinline__ uint32_t index_of<int32_t>(const int32_t* p, int64_t i) { return static_cast<uint32_t>(p[i]); }
+template <> __device__ __forceinline__ uint32_t index_of<uint8_t>(const uint8_t* p, int64_t i) { return p[i]; }
+struct Bf16Tag { uint16_t v; };
+struct Fp16Tag { uint16_t v; };
+template <> __device__ __forceinline__ uint32_t index_of<Bf16Tag>(const Bf16Tag* p, int64_t i) {
+    float f = bf16_bits_to_float(p[i].v);
+    return (f != f) ? 0u : static_cast<uint32_t>(static_cast<int>(f));
+}
+template <> __device__ __forceinline__ uint32_t index_of<Fp16Tag>(const Fp16Tag* p, int64_t i) {
+    float f = fp16_bits_to_float(p[i].v);
+    return (f != f) ? 0u : static_cast<uint32_t>(static_cast<int>(f));
+}
+
+template <typename IT, int BITS>
+__global__ void encode_kernel(const IT* __restrict__ idx, int64_t nbytes, uint8_t* __restrict__ out) {
+    constexpr int dpe = 8 / BITS;
+    constexpr uint32_t m = (1u << BITS) - 1u;
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < nbytes;
+         i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+        uint32_t byte = 0;
+#pragma unroll
+        for (int k = 0; k < dpe; ++k) byte |= (index_of<IT>(idx, i * dpe + k) & m) << (BITS * (dpe - 1 - k));
+        out[i] = static_cast<uint8_t>(byte);
+    }
+}
+
+template <typename IT>
+static int run_encode(const void* idx, int64_t nbytes, int bits, uint8_t* out, hipStream_t st) {
+    int64_t blocks = (nbytes + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    if (bits == 1)
+        hipLaunchKernelGGL((encode_kernel<IT, 1>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st,
+                           static_cast<const IT*>(idx), nbytes, out);
+    else
+        hipLaunchKernelGGL((encode_kernel<IT, 2>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st,
+                           static_cast<const IT*>(idx), nbytes, out);
+    CQ_LAUNCH_CHECK();
+    return CQ_OK;
+}
+
+}  // namespace cq
+
+extern "C" {
+
+size_t cq_quantize_pack_workspace(int B, int T, int H, int D) {
+    if (B < 1 || T < 1 || H < 1 || D < 1) return 0;
+    return static_cast<size_t>(B) * H * cq::pick_chunks(B, T, H) * 2 * D * sizeof(float);
+}
+
+int cq_quantize_pack(const void* x, int dtype, int B, int T, int H, int D, int64_t stride_b, int64_t stride_t,
+                     int64_t stride_h, int bits, float clip, uint8_t* codes, void* scale, void* zero,
+                     void* workspace, size_t workspace_bytes, cq_stream_t stream) {
+    if (!codes) return CQ_ERR_NULL;
+    return cq::quant_entry(x, dtype, B, T, H, D, stride_b, stride_t, stride_h, bits, clip, codes, nullptr, scale,
+                           zero, workspace, workspace_bytes, stream);
+}
+
+int cq_quant(const void* x, int dtype, int B, int T, int H, int D, int64_t stride_b, int64_t stride_t,
+             int64_t stride_h, int bits, float clip, void* x_q, void* scale, void* zero, void* workspace,
+             size_t workspace_bytes, cq_stream_t stream) {
+    if (!x_q) return CQ_ERR_NULL;
+    return cq::quant_entry(x, dtype, B, T, H, D, stride_b, stride_t, stride_h, bits, clip, nullptr, x_q, scale,
+                           zero, workspace, workspace_bytes, stream);
+}
+
+int cq_encode(const void* idx, int idx_dtype, int64_t rows, int D, int bits, uint8_t* out, cq_stream_t stream) {
+    if (!idx || !out) return CQ_ERR_NULL;
+    if (bits != 1 && bits != 2) return CQ_ERR_UNSUPPORTED;
+    if (rows < 0 || D < 1 || (D % (8 / bits)) != 0) return CQ_ERR_SHAPE;
+    if (rows == 0) return CQ_OK;
+    const int64_t nbytes = rows * (D * bits / 8);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (idx_dtype) {
+        case CQ_I64: return cq::run_encode<int64_t>(idx, nbytes, bits, out, s);
+        case CQ_I32: return cq::run_encode<int32_t>(idx, nbytes, bits, out, s);
+        case CQ_U8: return cq::run_encode<uint8_t>(idx, nbytes, bits, out, s);
+        case CQ_BF16: return cq::run_encode<cq::Bf16Tag>(idx, nbytes, bits, out, s);
+        case CQ_FP16: return cq::run_encode<cq::Fp16Tag>(idx, nbytes, bits, out, s);
+        default: return CQ_ERR_DTYPE;
+    }
+}
+
+}  // extern "C"

@@ -1,0 +1,187 @@
+"""Fused operators of the MI355X CalibQuant path (torch tensors in, HIP out).
+
+`quantize_pack` replaces the prefill chain quant -> LUT indices -> encode of the
+reference (calibquant.py:24-42, patch_internvl.py:318-329, calibquant.py:114-137)
+and `decode_attn` replaces its decode branch (patch_internvl.py:344-436).  Both
+call the C-ABI library on torch's current stream; torch only owns the memory."""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+_DT = {torch.bfloat16: _lib.CQ_BF16, torch.float16: _lib.CQ_FP16, torch.float32: _lib.CQ_FP32,
+       torch.int64: _lib.CQ_I64, torch.int32: _lib.CQ_I32, torch.uint8: _lib.CQ_U8}
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _need_gpu(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise _lib.CalibQuantError(f"{name} must live on the GPU (got {t.device}); there is no CPU path")
+
+
+def _storage_dtype(t: torch.Tensor, name: str) -> int:
+    if t.dtype not in (torch.bfloat16, torch.float16):
+        raise _lib.CalibQuantError(f"{name}: dtype {t.dtype} not supported (bf16 / fp16 only)")
+    return _DT[t.dtype]
+
+
+def _workspace(nbytes: int, device) -> Optional[torch.Tensor]:
+    if nbytes == 0:
+        return None
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
+def quantize_pack(x: torch.Tensor, bits: int, clip: float) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Per-channel min-max quantise and bit-pack one K or V tensor.
+
+    x: (B, T, H, D) view (any b/t/h strides, D contiguous), bf16 or fp16.
+    Returns codes uint8 (B, H, T, D*bits/8), scale (B, H, D), zero (B, H, D)."""
+    _need_gpu(x, "x")
+    dt = _storage_dtype(x, "x")
+    if x.dim() != 4 or x.stride(3) != 1:
+        raise _lib.CalibQuantError("x must be (B, T, H, D) with a contiguous last axis")
+    B, T, H, D = x.shape
+    lib = _lib.load()
+    codes = torch.empty((B, H, T, D * bits // 8), dtype=torch.uint8, device=x.device)
+    scale = torch.empty((B, H, D), dtype=x.dtype, device=x.device)
+    zero = torch.empty((B, H, D), dtype=x.dtype, device=x.device)
+    ws = _workspace(lib.cq_quantize_pack_workspace(B, T, H, D), x.device)
+    with torch.cuda.device(x.device):
+        rc = lib.cq_quantize_pack(x.data_ptr(), dt, B, T, H, D, x.stride(0), x.stride(1), x.stride(2),
+                                  bits, float(clip), codes.data_ptr(), scale.data_ptr(), zero.data_ptr(),
+                                  ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
+                                  _stream(x))
+    _lib.check(rc, "cq_quantize_pack")
+    return codes, scale, zero
+
+
+def quant_codes(x: torch.Tensor, bits: int, clip: float):
+    """The unfused quantiser: x (B, T, H, D) -> (x_q (B, T, H, D) of x.dtype
+    holding the integer codes, scale (B, 1, H, D), zero (B, 1, H, D))."""
+    _need_gpu(x, "x")
+    dt = _storage_dtype(x, "x")
+    if x.dim() != 4 or x.stride(3) != 1:
+        raise _lib.CalibQuantError("x must be (B, T, H, D) with a contiguous last axis")
+    B, T, H, D = x.shape
+    lib = _lib.load()
+    xq = torch.empty((B, T, H, D), dtype=x.dtype, device=x.device)
+    scale = torch.empty((B, 1, H, D), dtype=x.dtype, device=x.device)
+    zero = torch.empty((B, 1, H, D), dtype=x.dtype, device=x.device)
+    ws = _workspace(lib.cq_quantize_pack_workspace(B, T, H, D), x.device)
+    with torch.cuda.device(x.device):
+        rc = lib.cq_quant(x.data_ptr(), dt, B, T, H, D, x.stride(0), x.stride(1), x.stride(2),
+                          bits, float(clip), xq.data_ptr(), scale.data_ptr(), zero.data_ptr(),
+                          ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0, _stream(x))
+    _lib.check(rc, "cq_quant")
+    return xq, scale, zero
+
+
+def encode_indices(idx: torch.Tensor, bits: int) -> torch.Tensor:
+    """Pack integer indices (..., D) into uint8 (..., D*bits/8), first index in the high bits."""
+    _need_gpu(idx, "idx")
+    if idx.dtype not in _DT or idx.dtype == torch.float32:
+        raise _lib.CalibQuantError(f"encode: dtype {idx.dtype} not supported")
+    idx = idx.contiguous()
+    D = idx.shape[-1]
+    rows = idx.numel() // D if D else 0
+    out = torch.empty((*idx.shape[:-1], D * bits // 8), dtype=torch.uint8, device=idx.device)
+    with torch.cuda.device(idx.device):
+        rc = _lib.load().cq_encode(idx.data_ptr(), _DT[idx.dtype], rows, D, bits, out.data_ptr(), _stream(idx))
+    _lib.check(rc, "cq_encode")
+    return out
+
+
+def lut_vecmat(kind: str, lut: torch.Tensor, a: torch.Tensor, enc: torch.Tensor, bits: int) -> torch.Tensor:
+    """kind 'qk': a (M, D), enc (M, T, D*bits/8) -> (M, T) fp16;
+    kind 'pv': a (M, T), enc (M, T, D*bits/8) -> (M, D) fp16."""
+    for t, n in ((lut, "lut"), (a, "a"), (enc, "enc")):
+        _need_gpu(t, n)
+    lut, a, enc = lut.contiguous(), a.contiguous(), enc.contiguous()
+    M, T, nb = enc.shape
+    D = nb * 8 // bits
+    out = torch.empty((M, T if kind == "qk" else D), dtype=torch.float16, device=a.device)
+    fn = _lib.load().cq_lut_vecmat_qk if kind == "qk" else _lib.load().cq_lut_vecmat_pv
+    with torch.cuda.device(a.device):
+        rc = fn(lut.data_ptr(), _DT[lut.dtype], a.data_ptr(), _DT[a.dtype], enc.data_ptr(), M, T, D, bits,
+                out.data_ptr(), _stream(a))
+    _lib.check(rc, f"cq_lut_vecmat_{kind}")
+    return out
+
+
+def decode_attn(q: torch.Tensor, codes_k: Optional[torch.Tensor], codes_v: Optional[torch.Tensor],
+                k_scale: Optional[torch.Tensor], k_zero: Optional[torch.Tensor],
+                v_scale: Optional[torch.Tensor], v_zero: Optional[torch.Tensor],
+                k_res: Optional[torch.Tensor], v_res: Optional[torch.Tensor],
+                sprompt_len: int = 0, bits: int = 1, calibrate: bool = True,
+                calib_off_max: float = -3.0, calib_off_min: float = 0.0,
+                mask: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                force_splits: int = 0) -> torch.Tensor:
+    """One decode-attention step over packed image K/V plus the fp residual window.
+
+    q (B, Hq, D); codes_* uint8 (B, Hkv, T, D*bits/8); *_scale, *_zero (B, Hkv, D);
+    k_res, v_res (B, Hkv, R, D) (any b/h/r strides); mask optional additive
+    (B, S + T + R - S) fp32 over the [sys | image | text] order.  Returns (B, Hq, D)."""
+    _need_gpu(q, "q")
+    dt = _storage_dtype(q, "q")
+    q = q.contiguous()
+    B, Hq, D = q.shape
+    a = _lib.DecodeArgs()
+    T = 0
+    Hkv = None
+    keep = [q]
+    if codes_k is not None and codes_k.shape[2] > 0:
+        for t in (codes_k, codes_v, k_scale, k_zero, v_scale, v_zero):
+            _need_gpu(t, "packed state")
+        codes_k, codes_v = codes_k.contiguous(), codes_v.contiguous()
+        k_scale, k_zero = k_scale.contiguous(), k_zero.contiguous()
+        v_scale, v_zero = v_scale.contiguous(), v_zero.contiguous()
+        for t in (k_scale, k_zero, v_scale, v_zero):
+            if t.dtype != q.dtype:
+                raise _lib.CalibQuantError("scale / zero-point dtype must match q")
+        Hkv, T = codes_k.shape[1], codes_k.shape[2]
+        a.codes_k, a.codes_v = codes_k.data_ptr(), codes_v.data_ptr()
+        a.k_scale, a.k_zero = k_scale.data_ptr(), k_zero.data_ptr()
+        a.v_scale, a.v_zero = v_scale.data_ptr(), v_zero.data_ptr()
+        keep += [codes_k, codes_v, k_scale, k_zero, v_scale, v_zero]
+    R = 0
+    if k_res is not None and k_res.shape[2] > 0:
+        _need_gpu(k_res, "k_res")
+        if k_res.dtype != q.dtype or v_res.dtype != q.dtype:
+            raise _lib.CalibQuantError("residual dtype must match q")
+        if k_res.stride(3) != 1 or v_res.stride(3) != 1 or k_res.stride() != v_res.stride():
+            k_res, v_res = k_res.contiguous(), v_res.contiguous()
+        Hkv, R = k_res.shape[1], k_res.shape[2]
+        a.k_res, a.v_res = k_res.data_ptr(), v_res.data_ptr()
+        a.res_stride_b, a.res_stride_h, a.res_stride_r = k_res.stride(0), k_res.stride(1), k_res.stride(2)
+        keep += [k_res, v_res]
+    if Hkv is None:
+        raise _lib.CalibQuantError("decode_attn needs packed tokens or residual rows")
+    if mask is not None:
+        _need_gpu(mask, "mask")
+        mask = mask.reshape(B, -1).to(torch.float32).contiguous()
+        if mask.shape[1] != T + R:
+            raise _lib.CalibQuantError(f"mask length {mask.shape[1]} != T + R = {T + R}")
+        a.mask, a.mask_stride_b = mask.data_ptr(), mask.stride(0)
+        keep.append(mask)
+    if out is None:
+        out = torch.empty_like(q)
+    a.q, a.out = q.data_ptr(), out.data_ptr()
+    a.dtype, a.B, a.Hq, a.Hkv, a.D, a.T, a.R = dt, B, Hq, Hkv, D, T, R
+    a.sprompt_len, a.bits = int(sprompt_len), int(bits)
+    a.calibrate, a.calib_off_max, a.calib_off_min = int(bool(calibrate)), float(calib_off_max), float(calib_off_min)
+    a.force_splits = int(force_splits)
+    lib = _lib.load()
+    ws = _workspace(lib.cq_decode_attn_workspace(C.byref(a)), q.device)
+    if ws is not None:
+        a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    with torch.cuda.device(q.device):
+        rc = lib.cq_decode_attn(C.byref(a), _stream(q))
+    _lib.check(rc, "cq_decode_attn")
+    return out

@@ -1,0 +1,154 @@
+/* calibquant_hip.h - C ABI of the MI355X (gfx950) CalibQuant kernels.
+ *
+ * Plain pointers and sizes only.  All pointers are device pointers unless the
+ * comment says otherwise.  No function allocates, frees or synchronises; every
+ * launch goes to `stream` (a hipStream_t passed as an opaque pointer, NULL =
+ * the default stream).  Return value: CQ_OK (0) or a negative CQ_ERR_* code;
+ * cq_strerror() names it and cq_last_hip_error() returns the hipError_t of the
+ * last failed runtime call made on the calling host thread.
+ *
+ * Storage dtypes: CQ_BF16 or CQ_FP16 (16-bit).  "Storage-dtype arithmetic"
+ * means fp32 compute with a round-to-nearest-even cast after every operation,
+ * which is how the reference's torch op chains behave on 16-bit tensors.
+ *
+ * Each entry point names the reference interface it replaces
+ * (paths relative to the reference checkout).
+ */
+#ifndef CALIBQUANT_HIP_H
+#define CALIBQUANT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* cq_stream_t; /* hipStream_t */
+
+enum cq_dtype { CQ_BF16 = 0, CQ_FP16 = 1, CQ_FP32 = 2, CQ_I64 = 3, CQ_I32 = 4, CQ_U8 = 5 };
+
+enum cq_status {
+    CQ_OK = 0,
+    CQ_ERR_NULL = -1,        /* a required pointer is NULL */
+    CQ_ERR_SHAPE = -2,       /* a dimension is out of the supported range */
+    CQ_ERR_DTYPE = -3,       /* dtype code not accepted by this entry point */
+    CQ_ERR_ALIGN = -4,       /* pointer or stride not 16-byte aligned */
+    CQ_ERR_WORKSPACE = -5,   /* workspace missing or too small */
+    CQ_ERR_LAUNCH = -6,      /* the HIP runtime reported an error */
+    CQ_ERR_UNSUPPORTED = -7  /* valid request that this build does not cover */
+};
+
+int cq_version(void);
+const char* cq_strerror(int status);
+int cq_last_hip_error(void);
+
+/* ------------------------------------------------------------------------
+ * Prefill: per-channel min-max quantise + bit-pack of one K or V tensor.
+ * Replaces the chain quant() -> LUT/index build -> encode():
+ *   calibquant.py:24-42 (quant, per_channel=True, post_scale=True),
+ *   patch_internvl.py:292,297 (call sites), :318-329 (LUT indices),
+ *   calibquant.py:114-137 (encode), patch_internvl.py:332,339.
+ *
+ * x      (B, T, H, D) view in storage dtype; element strides stride_b/t/h,
+ *        D contiguous.  D in {64, 128, 256}; strides multiples of 8.
+ * bits   1 or 2.  clip = the reference's SCALE_K / SCALE_V factor.
+ * codes  uint8 (B, H, T, D*bits/8), first channel in the most significant bits.
+ * scale, zero   storage dtype, (B, H, D); bit-identical to the reference's
+ *        storage-dtype arithmetic, including scale 0 / zero -inf|NaN for a
+ *        constant channel (whose codes are 0, as in the reference).
+ * workspace     cq_quantize_pack_workspace(B, T, H, D) bytes, 16-byte aligned.
+ * Inputs must not contain NaN. */
+size_t cq_quantize_pack_workspace(int B, int T, int H, int D);
+int cq_quantize_pack(const void* x, int dtype, int B, int T, int H, int D,
+                     int64_t stride_b, int64_t stride_t, int64_t stride_h,
+                     int bits, float clip,
+                     uint8_t* codes, void* scale, void* zero,
+                     void* workspace, size_t workspace_bytes, cq_stream_t stream);
+
+/* quant() itself, for callers that keep the reference's unfused call sequence
+ * (calibquant.py:24-42 with per_channel=True, post_scale=True).  x_q is a
+ * contiguous (B, T, H, D) tensor of storage dtype holding the integer codes
+ * (NaN where the reference yields NaN); scale, zero as above. */
+int cq_quant(const void* x, int dtype, int B, int T, int H, int D,
+             int64_t stride_b, int64_t stride_t, int64_t stride_h,
+             int bits, float clip,
+             void* x_q, void* scale, void* zero,
+             void* workspace, size_t workspace_bytes, cq_stream_t stream);
+
+/* encode(): pack `rows` rows of D integer indices, 8/bits per byte,
+ * first index in the most significant bits (calibquant.py:114-137).
+ * idx_dtype: CQ_I64, CQ_I32, CQ_U8, or CQ_BF16/CQ_FP16 numbers holding
+ * integers.  Only the low `bits` bits of each index are kept. */
+int cq_encode(const void* idx, int idx_dtype, int64_t rows, int D, int bits,
+              uint8_t* out, cq_stream_t stream);
+
+/* fused_kernel(): c[m, t] = sum_d a[m, d] * lut[code[m, t, d]], fp32
+ * accumulation, fp16 output (calibquant.py:54-111).  a: (M, D) in a_dtype
+ * (CQ_BF16/CQ_FP16/CQ_FP32); enc: (M, T, D*bits/8); lut: 2^bits entries in
+ * lut_dtype; out: (M, T) fp16. */
+int cq_lut_vecmat_qk(const void* lut, int lut_dtype, const void* a, int a_dtype,
+                     const uint8_t* enc, int64_t M, int T, int D, int bits,
+                     void* out_fp16, cq_stream_t stream);
+
+/* fused_kernel_wv(): c[m, d] = sum_t a[m, t] * lut[code[m, t, d]], fp32
+ * accumulation, fp16 output (calibquant.py:192-276).  a: (M, T);
+ * enc: (M, T, D*bits/8); out: (M, D) fp16. */
+int cq_lut_vecmat_pv(const void* lut, int lut_dtype, const void* a, int a_dtype,
+                     const uint8_t* enc, int64_t M, int T, int D, int bits,
+                     void* out_fp16, cq_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Decode: one fused attention step over packed image K/V plus the
+ * full-precision residual window.  Replaces the whole decode branch
+ * patch_internvl.py:344-436: repeat_kv copies (:352-353, 361-362), residual
+ * logits (:365-366), post-scaled image logits through fused_kernel
+ * (:369-373), calibration (:376-385), concatenation [sys | image | text]
+ * (:388), additive mask (:404-410), softmax (:413), fused_kernel_wv and value
+ * post-scaling (:418-425), residual outputs and their sum (:428-436).
+ * Arithmetic is fp32 with one final rounding to the storage dtype. */
+typedef struct cq_decode_args {
+    /* query, (B, Hq, D) contiguous, storage dtype; D must be 128 */
+    const void* q;
+    /* packed codes, uint8 (B, Hkv, T, D*bits/8) contiguous */
+    const uint8_t* codes_k;
+    const uint8_t* codes_v;
+    /* per-channel statistics, storage dtype, (B, Hkv, D) contiguous */
+    const void* k_scale;
+    const void* k_zero;
+    const void* v_scale;
+    const void* v_zero;
+    /* residual window, storage dtype, (B, Hkv, R, D) with element strides
+     * res_stride_b/h/r (D contiguous; strides multiples of 8).  Rows
+     * [0, sprompt_len) precede the image block, the rest follow it. */
+    const void* k_res;
+    const void* v_res;
+    int64_t res_stride_b, res_stride_h, res_stride_r;
+    /* optional additive mask, fp32, row b at mask + b*mask_stride_b, indexed
+     * over the [sys | image | text] order (length sprompt_len + T + R - sprompt_len) */
+    const float* mask;
+    int64_t mask_stride_b;
+    /* output, (B, Hq, D) contiguous, storage dtype */
+    void* out;
+    /* cq_decode_attn_workspace() bytes, 16-byte aligned; may be NULL if that is 0 */
+    void* workspace;
+    size_t workspace_bytes;
+    int dtype;          /* CQ_BF16 or CQ_FP16 */
+    int B, Hq, Hkv, D;
+    int T;              /* packed (image) tokens, may be 0 */
+    int R;              /* residual rows, may be 0 (T + R > 0) */
+    int sprompt_len;    /* 0 <= sprompt_len <= R */
+    int bits;           /* 1 or 2 */
+    int calibrate;      /* non-zero: apply the logit calibration */
+    float calib_off_max;   /* reference: -3 */
+    float calib_off_min;   /* reference:  0 */
+    int force_splits;   /* 0 = choose; >0 = split the T axis into this many chunks */
+} cq_decode_args;
+
+size_t cq_decode_attn_workspace(const cq_decode_args* args);
+int cq_decode_attn(const cq_decode_args* args, cq_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CALIBQUANT_HIP_H */

@@ -1,0 +1,163 @@
+"""GPU parity of the fused decode-attention kernel against the fp32
+dequant-attention oracle computed from the same packed codes and statistics.
+Tolerance (stated by the task): 1e-2 max-abs, 1e-3 mean-abs."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import cq_oracle as O
+from tests.util import case_to_gpu, make_case, to_np
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, MEAN_ABS = 1e-2, 1e-3
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from calibquant_amd import ops
+    return ops
+
+
+def _run(ops, c, dtype, S, bits, mask=None, **kw):
+    g = case_to_gpu(c, dtype)
+    m = None if mask is None else torch.from_numpy(mask.astype(np.float32)).cuda()
+    out = ops.decode_attn(g["q"], g["ck"], g["cv"], g["sk"], g["zk"], g["sv"], g["zv"], g["kr"], g["vr"],
+                          sprompt_len=S, bits=bits, mask=m, **kw)
+    torch.cuda.synchronize()
+    return to_np(out)
+
+
+def _oracle(c, S, bits, mask=None, **kw):
+    kr = c["kr"] if c["kr"].shape[2] else None
+    vr = c["vr"] if c["vr"].shape[2] else None
+    return O.decode_attention(c["q"], c["ck"], c["cv"], c["sk"], c["zk"], c["sv"], c["zv"], kr, vr, S, bits,
+                              mask=mask, **kw)
+
+
+def _check(got, want):
+    err = np.abs(got - want)
+    assert np.isfinite(got).all()
+    assert err.max() < MAX_ABS, f"max-abs {err.max():.3e}"
+    assert err.mean() < MEAN_ABS, f"mean-abs {err.mean():.3e}"
+
+
+CASES = [
+    # B, Hq, Hkv, T, R, S
+    (2, 32, 8, 3328, 128, 0),      # InternVL2.5-8B layer shape, small batch
+    (1, 32, 8, 1024, 0, 0),        # CPU-reference configuration: no residual
+    (2, 32, 8, 777, 60, 41),       # ragged T, system prompt of the reference (41 rows)
+    (1, 8, 8, 130, 5, 2),          # MHA-like: one q head per kv head
+    (1, 16, 8, 259, 70, 10),       # two q heads per kv head
+    (1, 48, 8, 1000, 33, 0),       # InternLM2-20B grouping: six q heads per kv head
+    (3, 32, 8, 1, 1, 1),           # single packed token
+]
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("bits", [1, 2])
+@pytest.mark.parametrize("case", CASES)
+def test_decode_attn_matches_oracle(ops, case, bits, dtype):
+    B, Hq, Hkv, T, R, S = case
+    print(f"case decode_attn {case} bits={bits} dtype={dtype}", flush=True)
+    c = make_case(B, Hq, Hkv, 128, T, R, bits, dtype, seed=T + R)
+    _check(_run(ops, c, dtype, S, bits), _oracle(c, S, bits))
+
+
+@pytest.mark.parametrize("bits", [1, 2])
+def test_decode_attn_without_calibration_and_custom_offsets(ops, bits):
+    c = make_case(2, 32, 8, 128, 500, 40, bits, "bf16", seed=9)
+    _check(_run(ops, c, "bf16", 7, bits, calibrate=False), _oracle(c, 7, bits, calibrate_logits=False))
+    _check(_run(ops, c, "bf16", 7, bits, calib_off_max=-1.5, calib_off_min=0.5),
+           _oracle(c, 7, bits, off_max=-1.5, off_min=0.5))
+
+
+@pytest.mark.parametrize("bits", [1, 2])
+def test_decode_attn_with_additive_mask(ops, bits):
+    B, Hq, Hkv, T, R, S = 2, 32, 8, 600, 50, 41
+    c = make_case(B, Hq, Hkv, 128, T, R, bits, "bf16", seed=4)
+    rng = np.random.default_rng(0)
+    mask = np.zeros((B, T + R), np.float32)
+    mask[0, :30] = -1e4                      # left padding inside the system prompt
+    mask[1, rng.integers(0, T + R, 100)] = -1e4
+    _check(_run(ops, c, "bf16", S, bits, mask=mask), _oracle(c, S, bits, mask=mask))
+
+
+def test_decode_attn_residual_only_and_strided_cache(ops):
+    """No packed tokens: plain attention over the fp window, read through a
+    view of a larger pre-allocated cache."""
+    B, Hq, Hkv, R = 2, 32, 8, 200
+    c = make_case(B, Hq, Hkv, 128, 64, R, 1, "bf16", seed=2)
+    g = case_to_gpu(c, "bf16")
+    cap = 512
+    kbuf = torch.zeros((B, Hkv, cap, 128), dtype=torch.bfloat16, device="cuda")
+    vbuf = torch.zeros_like(kbuf)
+    kbuf[:, :, :R] = g["kr"]
+    vbuf[:, :, :R] = g["vr"]
+    out = ops.decode_attn(g["q"], None, None, None, None, None, None, kbuf[:, :, :R], vbuf[:, :, :R])
+    want = O.decode_attention(c["q"], c["ck"][:, :, :0], c["cv"][:, :, :0], c["sk"], c["zk"], c["sv"], c["zv"],
+                              c["kr"], c["vr"], 0, 1)
+    _check(to_np(out), want)
+    out2 = ops.decode_attn(g["q"], g["ck"], g["cv"], g["sk"], g["zk"], g["sv"], g["zv"],
+                           kbuf[:, :, :R], vbuf[:, :, :R], sprompt_len=41)
+    _check(to_np(out2), _oracle(c, 41, 1))
+
+
+@pytest.mark.parametrize("bits", [1, 2])
+@pytest.mark.parametrize("splits", [2, 5])
+def test_decode_attn_split_path_matches_fused_path(ops, bits, splits):
+    B, Hq, Hkv, T, R, S = 1, 32, 8, 2000, 70, 3
+    c = make_case(B, Hq, Hkv, 128, T, R, bits, "bf16", seed=8)
+    want = _oracle(c, S, bits)
+    _check(_run(ops, c, "bf16", S, bits, force_splits=splits), want)
+    rng = np.random.default_rng(1)
+    mask = np.where(rng.random((B, T + R)) < 0.1, -1e4, 0.0).astype(np.float32)
+    _check(_run(ops, c, "bf16", S, bits, mask=mask, force_splits=splits), _oracle(c, S, bits, mask=mask))
+
+
+def test_decode_attn_long_context_auto_split(ops):
+    """KV 32768 at batch 1: the chunked path (min/max launch, main launch, merge)."""
+    B, Hq, Hkv, T, R = 1, 32, 8, 32768, 16
+    c = make_case(B, Hq, Hkv, 128, T, R, 1, "bf16", seed=12)
+    _check(_run(ops, c, "bf16", 0, 1), _oracle(c, 0, 1))
+
+
+def test_decode_attn_degenerate_range_and_peaked_softmax(ops):
+    """All packed keys identical (logit range 0) and a residual row that takes
+    nearly all the probability mass."""
+    c = make_case(1, 32, 8, 128, 256, 8, 1, "bf16", seed=6)
+    c["ck"][:] = c["ck"][:, :, :1]
+    c["kr"][:, :, 3] = O.round_to(c["q"].reshape(1, 8, 4, 128)[:, :, 0] * 4.0, "bf16")
+    _check(_run(ops, c, "bf16", 0, 1), _oracle(c, 0, 1))
+
+
+def test_decode_attn_full_batch_properties(ops):
+    """Batch 64, KV 3328 + 128 (the benchmark shape): every batch row is an
+    independent problem, so (a) a batch built by repeating one row gives
+    identical outputs per row, and (b) rows 0..1 equal the oracle."""
+    B, Hq, Hkv, T, R = 64, 32, 8, 3328, 128
+    c = make_case(2, Hq, Hkv, 128, T, R, 1, "bf16", seed=20, outlier_kind="student")
+    g = case_to_gpu(c, "bf16")
+    rep = {k: torch.cat([v] * (B // 2), 0) for k, v in g.items()}
+    out = ops.decode_attn(rep["q"], rep["ck"], rep["cv"], rep["sk"], rep["zk"], rep["sv"], rep["zv"],
+                          rep["kr"], rep["vr"])
+    torch.cuda.synchronize()
+    assert torch.equal(out[0::2], out[0:1].expand(B // 2, -1, -1))
+    assert torch.equal(out[1::2], out[1:2].expand(B // 2, -1, -1))
+    _check(to_np(out[:2]), _oracle(c, 0, 1))
+
+
+def test_decode_attn_rejects_bad_arguments(ops):
+    from calibquant_amd._lib import CalibQuantError
+    c = make_case(1, 32, 8, 128, 64, 8, 1, "bf16", seed=1)
+    g = case_to_gpu(c, "bf16")
+    with pytest.raises(CalibQuantError):
+        ops.decode_attn(g["q"].float(), g["ck"], g["cv"], g["sk"], g["zk"], g["sv"], g["zv"], g["kr"], g["vr"])
+    with pytest.raises(CalibQuantError):
+        ops.decode_attn(g["q"], g["ck"], g["cv"], g["sk"], g["zk"], g["sv"], g["zv"], g["kr"], g["vr"],
+                        sprompt_len=9)
+    with pytest.raises(CalibQuantError):
+        ops.decode_attn(g["q"].cpu(), g["ck"], g["cv"], g["sk"], g["zk"], g["sv"], g["zv"], g["kr"], g["vr"])
+    with pytest.raises(CalibQuantError):
+        ops.decode_attn(g["q"][:, :, :64].contiguous(), g["ck"], g["cv"], g["sk"], g["zk"], g["sv"], g["zv"],
+                        g["kr"], g["vr"])
