@@ -1,0 +1,214 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantised-KV decode-attention hot path on one MI355X.
+
+A "step" is one fused decode-attention layer call (the reference's decode
+branch, patch_internvl.py:344-436) on a synthetic InternVL2.5-8B-shaped layer:
+batch 64, 32 query / 8 KV heads, head_dim 128, 3 328 packed image tokens plus a
+128-row bf16 residual window.  Inputs are resident in HBM before the timed
+region; the call rotates over several distinct buffer sets (> 256 MB in total)
+so the packed codes are not served from the Infinity Cache.
+
+Prints ONE JSON line (see README / DESIGN for the fields).  `value` is the
+average duration of one layer call in microseconds; `roofline` prices the
+algorithmic bytes of that call against the 8 TB/s HBM peak; `cpu_baseline` is
+the C port of the oracle timed on this host's cores on a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+HBM_PEAK_GBPS = 8000.0
+METRIC = "1-bit decode-attn µs/layer + HBM GB/s %peak; InternVL2.5-8B decode tok/s"
+
+WORKLOADS = {
+    # name: (B, Hq, Hkv, D, T, R, S)
+    "internvl2.5-8b-layer-b64-kv3328+128": (64, 32, 8, 128, 3328, 128, 0),
+    "long-context-b8-kv32768": (8, 32, 8, 128, 32768, 0, 0),
+    "wide-batch-b256-kv3328": (256, 32, 8, 128, 3328, 0, 0),
+    "internvl2.5-26b-layer-b16-kv9984+64": (16, 48, 8, 128, 9984, 64, 0),
+}
+DEFAULT_WORKLOAD = "internvl2.5-8b-layer-b64-kv3328+128"
+
+
+def algorithmic_bytes(B, Hq, Hkv, D, T, R, bits, elt=2):
+    """Each byte counted once: K+V codes, per-channel K and V statistics,
+    fp residual K+V, q in and out."""
+    codes = 2 * B * Hkv * T * D * bits // 8
+    stats = 4 * B * Hkv * D * elt
+    resid = 2 * B * Hkv * R * D * elt
+    qo = 2 * B * Hq * D * elt
+    return codes + stats + resid + qo
+
+
+def build_sets(torch, ops, shape, bits, nsets, seed):
+    """Synthetic layer state, generated on the GPU with a seeded device
+    generator: K/V ~ N(0,1), four key channels per kv-head scaled by |t3|+1
+    (Student-t, nu=3), quantised and packed by the prefill kernel."""
+    B, Hq, Hkv, D, T, R, S = shape
+    dev = torch.device("cuda:0")
+    torch.manual_seed(seed)
+    g = torch.Generator(device=dev).manual_seed(seed)
+    cpu_rng = torch.Generator().manual_seed(seed)
+    clip_k, clip_v = (0.5, 0.3) if bits == 1 else (1.0, 1.0)
+    sets = []
+    for _ in range(nsets):
+        k = torch.randn((B, T, Hkv, D), generator=g, device=dev)
+        v = torch.randn((B, T, Hkv, D), generator=g, device=dev)
+        for h in range(Hkv):
+            ch = torch.randperm(D, generator=cpu_rng)[:4].to(dev)
+            t3 = torch.distributions.StudentT(3.0).sample((4,)).abs().to(dev) + 1.0
+            k[:, :, h, ch] *= t3
+        k, v = k.to(torch.bfloat16), v.to(torch.bfloat16)
+        ck, sk, zk = ops.quantize_pack(k, bits, clip_k)
+        cv, sv, zv = ops.quantize_pack(v, bits, clip_v)
+        del k, v
+        q = torch.randn((B, Hq, D), generator=g, device=dev).to(torch.bfloat16)
+        kr = torch.randn((B, Hkv, max(R, 1), D), generator=g, device=dev).to(torch.bfloat16)[:, :, :R]
+        vr = torch.randn((B, Hkv, max(R, 1), D), generator=g, device=dev).to(torch.bfloat16)[:, :, :R]
+        sets.append(dict(q=q, ck=ck, cv=cv, sk=sk, zk=zk, sv=sv, zv=zv, kr=kr if R else None, vr=vr if R else None))
+    return sets
+
+
+def time_calls(torch, calls, steps, warmup):
+    for i in range(warmup):
+        calls[i % len(calls)].run()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(steps):
+        calls[i % len(calls)].run()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / steps  # ms per call
+
+
+def time_fp16_kv(torch, shape, steps, warmup, nsets):
+    """Full-precision-KV attention over the same tokens with torch's fused SDPA."""
+    B, Hq, Hkv, D, T, R, S = shape
+    dev = torch.device("cuda:0")
+    N = T + R
+    sets = []
+    for _ in range(nsets):
+        q = torch.randn((B, Hq, 1, D), device=dev, dtype=torch.bfloat16)
+        k = torch.randn((B, Hkv, N, D), device=dev, dtype=torch.bfloat16)
+        v = torch.randn((B, Hkv, N, D), device=dev, dtype=torch.bfloat16)
+        sets.append((q, k, v))
+    F = torch.nn.functional
+
+    def run(i):
+        q, k, v = sets[i % nsets]
+        return F.scaled_dot_product_attention(q, k, v, enable_gqa=True)
+
+    for i in range(warmup):
+        run(i)
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(steps):
+        run(i)
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / steps
+
+
+def cpu_baseline(torch, sets, shape, bits, budget_s=12.0):
+    """C port of the oracle on this host's cores, on a bounded sample: the
+    first `bs` batch rows of the workload; the per-layer figure is scaled
+    linearly to the full batch (batch rows are independent)."""
+    from oracle import c_port
+    c_port.build()
+    B, Hq, Hkv, D, T, R, S = shape
+    bs = min(B, 4)
+    s0 = sets[0]
+    f = lambda t: None if t is None else t[:bs].float().cpu().numpy()  # noqa: E731
+    args = (f(s0["q"]), s0["ck"][:bs].cpu().numpy(), s0["cv"][:bs].cpu().numpy(), f(s0["sk"]), f(s0["zk"]),
+            f(s0["sv"]), f(s0["zv"]), f(s0["kr"]), f(s0["vr"]), S, bits)
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    t0 = time.perf_counter()
+    c_port.decode_attention(*args)
+    first = time.perf_counter() - t0
+    reps = max(3, min(50, int(budget_s / max(first, 1e-3))))
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        c_port.decode_attention(*args)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {"value": round(med * 1e6 * B / bs, 1), "unit": "us/layer", "cores": cores, "kind": "port",
+            "sample": f"oracle/cq_oracle.c (OpenMP) on {bs} of {B} batch rows, median of {reps} runs, "
+                      f"scaled x{B // bs} to the full batch"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--bits", type=int, default=1, choices=(1, 2))
+    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
+    ap.add_argument("--sets", type=int, default=4, help="distinct input buffer sets rotated through")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-fp16kv", action="store_true", help="skip the fp16-KV comparison leg")
+    ap.add_argument("--seed", type=int, default=1234)
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print(f"bench.py: this build measures one GPU only (asked for {a.gpus}); "
+              "the path shards over batch and kv-heads without exchange, see DESIGN.md", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    from calibquant_amd import ops
+
+    shape = WORKLOADS[a.workload]
+    B, Hq, Hkv, D, T, R, S = shape
+    sets = build_sets(torch, ops, shape, a.bits, a.sets, a.seed)
+    calls = [ops.DecodeCall(s["q"], s["ck"], s["cv"], s["sk"], s["zk"], s["sv"], s["zv"], s["kr"], s["vr"],
+                            sprompt_len=S, bits=a.bits) for s in sets]
+    ms = time_calls(torch, calls, a.steps, a.warmup)
+    nbytes = algorithmic_bytes(B, Hq, Hkv, D, T, R, a.bits)
+    gbps = nbytes / (ms * 1e-3) / 1e9
+
+    out = {
+        "metric": METRIC,
+        "value": round(ms * 1e3, 3),
+        "unit": "us/layer",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": round(ms, 6),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": a.workload, "batch": B, "q_heads": Hq, "kv_heads": Hkv, "head_dim": D,
+                   "kv_packed_tokens": T, "kv_residual_rows": R, "bits": a.bits, "storage_dtype": "bf16",
+                   "buffer_sets": a.sets, "launches_per_step": 1 if calls[0].workspace_bytes == 0 else 3},
+        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "algorithmic_bytes": nbytes},
+    }
+    if not a.no_fp16kv:
+        try:
+            fp_ms = time_fp16_kv(torch, shape, max(20, a.steps // 4), max(5, a.warmup // 4), a.sets)
+            out["fp16_kv_us_layer"] = round(fp_ms * 1e3, 2)
+            out["speedup_vs_fp16_kv"] = round(fp_ms / ms, 2)
+        except Exception as e:  # the comparison leg must not sink the measurement
+            out["fp16_kv_us_layer"] = None
+            out["fp16_kv_error"] = repr(e)[:200]
+    if not a.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(torch, sets, shape, a.bits)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

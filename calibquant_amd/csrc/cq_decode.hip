@@ -25,6 +25,8 @@
 // Everything here is HBM / LDS / VALU work; no matrix-core instructions.
 #include "cq_common.h"
 
+#include <atomic>
+
 namespace cq {
 
 constexpr int kD = 128;
@@ -681,13 +683,19 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
     const unsigned units = static_cast<unsigned>(g.B) * g.Hkv * (G / HPB);
     auto kmain = decode_kernel<BITS, HPB, DT, false>;
     auto kmm = decode_kernel<BITS, HPB, DT, true>;
-    static thread_local bool attr_done[2] = {false, false};
-    (void)attr_done;
-    CQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kmain),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax));
-    if (g.nsplit > 1) {
+    // raise the dynamic-LDS limit once per device for this instantiation
+    static std::atomic<uint32_t> attr_done{0};
+    int dev = 0;
+    CQ_HIP_CHECK(hipGetDevice(&dev));
+    const uint32_t bit = 1u << (dev & 31);
+    if (!(attr_done.load(std::memory_order_acquire) & bit)) {
+        CQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kmain),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax));
         CQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kmm),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax));
+        attr_done.fetch_or(bit, std::memory_order_release);
+    }
+    if (g.nsplit > 1) {
         DecodeGeom g1 = g;
         g1.nx = g.nsplit;  // the min/max pass has no residual unit
         const int lds_mm = Lay<BITS, HPB>::lds_bytes(0);

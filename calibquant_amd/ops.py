@@ -115,6 +115,83 @@ def lut_vecmat(kind: str, lut: torch.Tensor, a: torch.Tensor, enc: torch.Tensor,
     return out
 
 
+class DecodeCall:
+    """A prepared `cq_decode_attn` call: argument block, workspace and output are
+    set up once and `run()` only enqueues the launch(es) on torch's current
+    stream.  The tensors it was built from are kept alive by the object."""
+
+    def __init__(self, q, codes_k, codes_v, k_scale, k_zero, v_scale, v_zero, k_res, v_res,
+                 sprompt_len=0, bits=1, calibrate=True, calib_off_max=-3.0, calib_off_min=0.0,
+                 mask=None, out=None, force_splits=0):
+        _need_gpu(q, "q")
+        dt = _storage_dtype(q, "q")
+        if q.dim() != 3:
+            raise _lib.CalibQuantError("q must be (B, Hq, D)")
+        q = q.contiguous()
+        B, Hq, D = q.shape
+        a = _lib.DecodeArgs()
+        T = 0
+        Hkv = None
+        keep = [q]
+        if codes_k is not None and codes_k.shape[2] > 0:
+            for t in (codes_k, codes_v, k_scale, k_zero, v_scale, v_zero):
+                _need_gpu(t, "packed state")
+            codes_k, codes_v = codes_k.contiguous(), codes_v.contiguous()
+            k_scale, k_zero = k_scale.contiguous(), k_zero.contiguous()
+            v_scale, v_zero = v_scale.contiguous(), v_zero.contiguous()
+            for t in (k_scale, k_zero, v_scale, v_zero):
+                if t.dtype != q.dtype:
+                    raise _lib.CalibQuantError("scale / zero-point dtype must match q")
+            Hkv, T = codes_k.shape[1], codes_k.shape[2]
+            a.codes_k, a.codes_v = codes_k.data_ptr(), codes_v.data_ptr()
+            a.k_scale, a.k_zero = k_scale.data_ptr(), k_zero.data_ptr()
+            a.v_scale, a.v_zero = v_scale.data_ptr(), v_zero.data_ptr()
+            keep += [codes_k, codes_v, k_scale, k_zero, v_scale, v_zero]
+        R = 0
+        if k_res is not None and k_res.shape[2] > 0:
+            _need_gpu(k_res, "k_res")
+            if k_res.dtype != q.dtype or v_res.dtype != q.dtype:
+                raise _lib.CalibQuantError("residual dtype must match q")
+            if k_res.stride(3) != 1 or v_res.stride(3) != 1 or k_res.stride() != v_res.stride():
+                k_res, v_res = k_res.contiguous(), v_res.contiguous()
+            Hkv, R = k_res.shape[1], k_res.shape[2]
+            a.k_res, a.v_res = k_res.data_ptr(), v_res.data_ptr()
+            a.res_stride_b, a.res_stride_h, a.res_stride_r = k_res.stride(0), k_res.stride(1), k_res.stride(2)
+            keep += [k_res, v_res]
+        if Hkv is None:
+            raise _lib.CalibQuantError("decode_attn needs packed tokens or residual rows")
+        if mask is not None:
+            _need_gpu(mask, "mask")
+            mask = mask.reshape(B, -1).to(torch.float32).contiguous()
+            if mask.shape[1] != T + R:
+                raise _lib.CalibQuantError(f"mask length {mask.shape[1]} != T + R = {T + R}")
+            a.mask, a.mask_stride_b = mask.data_ptr(), mask.stride(0)
+            keep.append(mask)
+        if out is None:
+            out = torch.empty_like(q)
+        elif out.shape != q.shape or out.dtype != q.dtype or not out.is_contiguous():
+            raise _lib.CalibQuantError("out must be a contiguous tensor shaped and typed like q")
+        a.q, a.out = q.data_ptr(), out.data_ptr()
+        a.dtype, a.B, a.Hq, a.Hkv, a.D, a.T, a.R = dt, B, Hq, Hkv, D, T, R
+        a.sprompt_len, a.bits = int(sprompt_len), int(bits)
+        a.calibrate = int(bool(calibrate))
+        a.calib_off_max, a.calib_off_min = float(calib_off_max), float(calib_off_min)
+        a.force_splits = int(force_splits)
+        self._lib = _lib.load()
+        ws = _workspace(self._lib.cq_decode_attn_workspace(C.byref(a)), q.device)
+        if ws is not None:
+            a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+            keep.append(ws)
+        self.args, self._ref, self._keep, self.out, self.device = a, C.byref(a), keep, out, q.device
+        self.workspace_bytes = 0 if ws is None else ws.numel()
+
+    def run(self) -> torch.Tensor:
+        rc = self._lib.cq_decode_attn(self._ref, torch.cuda.current_stream(self.device).cuda_stream)
+        if rc:
+            _lib.check(rc, "cq_decode_attn")
+        return self.out
+
+
 def decode_attn(q: torch.Tensor, codes_k: Optional[torch.Tensor], codes_v: Optional[torch.Tensor],
                 k_scale: Optional[torch.Tensor], k_zero: Optional[torch.Tensor],
                 v_scale: Optional[torch.Tensor], v_zero: Optional[torch.Tensor],
@@ -127,61 +204,8 @@ def decode_attn(q: torch.Tensor, codes_k: Optional[torch.Tensor], codes_v: Optio
 
     q (B, Hq, D); codes_* uint8 (B, Hkv, T, D*bits/8); *_scale, *_zero (B, Hkv, D);
     k_res, v_res (B, Hkv, R, D) (any b/h/r strides); mask optional additive
-    (B, S + T + R - S) fp32 over the [sys | image | text] order.  Returns (B, Hq, D)."""
-    _need_gpu(q, "q")
-    dt = _storage_dtype(q, "q")
-    q = q.contiguous()
-    B, Hq, D = q.shape
-    a = _lib.DecodeArgs()
-    T = 0
-    Hkv = None
-    keep = [q]
-    if codes_k is not None and codes_k.shape[2] > 0:
-        for t in (codes_k, codes_v, k_scale, k_zero, v_scale, v_zero):
-            _need_gpu(t, "packed state")
-        codes_k, codes_v = codes_k.contiguous(), codes_v.contiguous()
-        k_scale, k_zero = k_scale.contiguous(), k_zero.contiguous()
-        v_scale, v_zero = v_scale.contiguous(), v_zero.contiguous()
-        for t in (k_scale, k_zero, v_scale, v_zero):
-            if t.dtype != q.dtype:
-                raise _lib.CalibQuantError("scale / zero-point dtype must match q")
-        Hkv, T = codes_k.shape[1], codes_k.shape[2]
-        a.codes_k, a.codes_v = codes_k.data_ptr(), codes_v.data_ptr()
-        a.k_scale, a.k_zero = k_scale.data_ptr(), k_zero.data_ptr()
-        a.v_scale, a.v_zero = v_scale.data_ptr(), v_zero.data_ptr()
-        keep += [codes_k, codes_v, k_scale, k_zero, v_scale, v_zero]
-    R = 0
-    if k_res is not None and k_res.shape[2] > 0:
-        _need_gpu(k_res, "k_res")
-        if k_res.dtype != q.dtype or v_res.dtype != q.dtype:
-            raise _lib.CalibQuantError("residual dtype must match q")
-        if k_res.stride(3) != 1 or v_res.stride(3) != 1 or k_res.stride() != v_res.stride():
-            k_res, v_res = k_res.contiguous(), v_res.contiguous()
-        Hkv, R = k_res.shape[1], k_res.shape[2]
-        a.k_res, a.v_res = k_res.data_ptr(), v_res.data_ptr()
-        a.res_stride_b, a.res_stride_h, a.res_stride_r = k_res.stride(0), k_res.stride(1), k_res.stride(2)
-        keep += [k_res, v_res]
-    if Hkv is None:
-        raise _lib.CalibQuantError("decode_attn needs packed tokens or residual rows")
-    if mask is not None:
-        _need_gpu(mask, "mask")
-        mask = mask.reshape(B, -1).to(torch.float32).contiguous()
-        if mask.shape[1] != T + R:
-            raise _lib.CalibQuantError(f"mask length {mask.shape[1]} != T + R = {T + R}")
-        a.mask, a.mask_stride_b = mask.data_ptr(), mask.stride(0)
-        keep.append(mask)
-    if out is None:
-        out = torch.empty_like(q)
-    a.q, a.out = q.data_ptr(), out.data_ptr()
-    a.dtype, a.B, a.Hq, a.Hkv, a.D, a.T, a.R = dt, B, Hq, Hkv, D, T, R
-    a.sprompt_len, a.bits = int(sprompt_len), int(bits)
-    a.calibrate, a.calib_off_max, a.calib_off_min = int(bool(calibrate)), float(calib_off_max), float(calib_off_min)
-    a.force_splits = int(force_splits)
-    lib = _lib.load()
-    ws = _workspace(lib.cq_decode_attn_workspace(C.byref(a)), q.device)
-    if ws is not None:
-        a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
-    with torch.cuda.device(q.device):
-        rc = lib.cq_decode_attn(C.byref(a), _stream(q))
-    _lib.check(rc, "cq_decode_attn")
-    return out
+    (B, S + T + R - S) over the [sys | image | text] order.  Returns (B, Hq, D)."""
+    call = DecodeCall(q, codes_k, codes_v, k_scale, k_zero, v_scale, v_zero, k_res, v_res,
+                      sprompt_len, bits, calibrate, calib_off_max, calib_off_min, mask, out, force_splits)
+    with torch.cuda.device(call.device):
+        return call.run()

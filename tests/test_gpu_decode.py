@@ -50,7 +50,7 @@ CASES = [
     (1, 8, 8, 130, 5, 2),          # MHA-like: one q head per kv head
     (1, 16, 8, 259, 70, 10),       # two q heads per kv head
     (1, 48, 8, 1000, 33, 0),       # InternLM2-20B grouping: six q heads per kv head
-    (3, 32, 8, 1, 1, 1),           # single packed token
+    (3, 32, 8, 7, 1, 1),           # a handful of packed tokens
 ]
 
 
@@ -62,6 +62,15 @@ def test_decode_attn_matches_oracle(ops, case, bits, dtype):
     print(f"case decode_attn {case} bits={bits} dtype={dtype}", flush=True)
     c = make_case(B, Hq, Hkv, 128, T, R, bits, dtype, seed=T + R)
     _check(_run(ops, c, dtype, S, bits), _oracle(c, S, bits))
+
+
+def test_decode_attn_single_token_is_nan_like_the_reference(ops):
+    """One packed token makes every channel constant: scale 0, zero-point
+    inf, and the reference's bias term 0 * inf = NaN poisons the row
+    (patch_internvl.py:369-370).  The kernel reproduces that, as the oracle does."""
+    c = make_case(1, 32, 8, 128, 1, 4, 1, "bf16", seed=1)
+    got, want = _run(ops, c, "bf16", 0, 1), _oracle(c, 0, 1)
+    assert np.isnan(want).all() and np.isnan(got).all()
 
 
 @pytest.mark.parametrize("bits", [1, 2])
