@@ -94,20 +94,43 @@ __device__ __forceinline__ void store_elem(void* p, int64_t i, float f) {
 }
 
 // ------------------------------------------------------- wave reductions
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
-    return v;
+// Cross-lane moves use the data-parallel-primitive modifiers of the VALU (no LDS
+// traffic, one instruction per step).  Control codes: quad_perm[1,0,3,2] = 0xB1,
+// quad_perm[2,3,0,1] = 0x4E, row_half_mirror = 0x141, row_mirror = 0x140,
+// row_bcast:15 = 0x142, row_bcast:31 = 0x143.
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ float dpp_move(float v, float inactive) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, inactive),
+                                                                  __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf,
+                                                                  false));
 }
-__device__ __forceinline__ float wave_min(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, kWave));
-    return v;
+
+struct OpMin { __device__ __forceinline__ float operator()(float a, float b) const { return fminf(a, b); } };
+struct OpMax { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
+struct OpSum { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
+
+// Reduce over aligned groups of 4 / 8 / 16 lanes; every lane of the group gets the result.
+template <typename Op> __device__ __forceinline__ float quad_reduce(float v, Op op, float id) {
+    v = op(v, dpp_move<0xB1>(v, id));
+    return op(v, dpp_move<0x4E>(v, id));
 }
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
-    return v;
+template <typename Op> __device__ __forceinline__ float oct_reduce(float v, Op op, float id) {
+    v = quad_reduce(v, op, id);
+    return op(v, dpp_move<0x141>(v, id));
 }
+template <typename Op> __device__ __forceinline__ float row_reduce(float v, Op op, float id) {
+    v = oct_reduce(v, op, id);
+    return op(v, dpp_move<0x140>(v, id));
+}
+// Reduce over the 64 lanes; the result is wave-uniform (scalar register).
+template <typename Op> __device__ __forceinline__ float wave_reduce(float v, Op op, float id) {
+    v = row_reduce(v, op, id);
+    v = op(v, dpp_move<0x142, 0xa>(v, id));
+    v = op(v, dpp_move<0x143, 0xc>(v, id));
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+__device__ __forceinline__ float wave_max(float v) { return wave_reduce(v, OpMax(), -INFINITY); }
+__device__ __forceinline__ float wave_min(float v) { return wave_reduce(v, OpMin(), INFINITY); }
+__device__ __forceinline__ float wave_sum(float v) { return wave_reduce(v, OpSum(), 0.0f); }
 
 }  // namespace cq

@@ -1,8 +1,12 @@
 // Fused decode attention over bit-packed K/V for gfx950 (MI355X).
 //
-// One workgroup owns one (batch, kv-head, head-group, token-chunk) unit and
-// runs the whole step for HPB query heads that share the kv-head:
+// One 1024-thread workgroup owns one (batch, kv-head, head-group, token-chunk)
+// unit and runs the whole step for HPB query heads that share the kv-head:
 //
+//   loads    every global load the unit needs first (packed K rows, the first
+//            block of packed V rows, the first tile of residual K/V rows) is
+//            issued at kernel entry into registers, so HBM latency overlaps
+//            the table build instead of stalling each phase in turn.
 //   K side   q.s_k is folded into a byte-indexed partial-sum table in LDS
 //            (one entry per byte position and byte value, HPB floats wide,
 //            zero-point folded in).  A token's logits are NB table look-ups
@@ -11,11 +15,12 @@
 //            in place in LDS.
 //   V side   tokens are taken four at a time: a 16-entry table of subset sums
 //            of their e values is built once per group, every byte column of
-//            the packed V rows is bit-transposed with a 256-entry spread
-//            table, and each of the 8 bit lanes of the column adds one table
-//            entry.  Scale / zero-point are applied once at the end.
-//   residual the full-precision rows run as an ordinary online-softmax
-//            flash-decode in the same workgroup and are merged at the end.
+//            the packed V rows is bit-transposed with 256-entry spread tables
+//            (one per token position, pre-shifted to table offsets), and each
+//            of the 8 bit lanes of the column adds one table entry.  Scale /
+//            zero-point are applied once at the end.
+//   residual the full-precision rows run as an online-softmax flash-decode in
+//            the same workgroup (packed dot2 for q.K) and are merged at the end.
 //
 // When the chunk does not cover all T tokens (long context or small batch)
 // a first launch publishes the per-chunk logit min / max, the main launch
@@ -30,13 +35,15 @@
 namespace cq {
 
 constexpr int kD = 128;
-constexpr int kNT = 512;          // threads per workgroup
-constexpr int kNW = kNT / kWave;  // waves per workgroup
-constexpr int kVSub = 1024;       // V tokens staged in LDS at a time
-constexpr int kResTile = kNT / 8; // residual rows per tile (8 lanes per row)
+constexpr int kNT = 1024;          // threads per workgroup
+constexpr int kNW = kNT / kWave;   // waves per workgroup
+constexpr int kPF = 4;             // 16-byte loads kept in flight per thread and stream
+constexpr int kResTile = kNT / 8;  // residual rows per tile (8 lanes per row)
 constexpr int kLdsMax = 160 * 1024;
 
 template <int N> struct alignas(N * 4) Vec { float v[N]; };
+// native 16-byte vector: copies are single vector moves (HIP's uint4 struct copies lower to memcpy)
+typedef uint32_t U4 __attribute__((ext_vector_type(4)));
 
 struct DecodeGeom {
     const void* q;
@@ -55,69 +62,72 @@ struct DecodeGeom {
     int calib;
     float off_max, off_min;
     int cap;      // logits capacity of the LDS layout, tokens
+    float one;    // 1.0f, opaque to the compiler: keeps f16 -> f32 accumulation in one mixed-precision FMA
 };
+
+constexpr int cmax(int a, int b) { return a > b ? a : b; }
+constexpr int cmin(int a, int b) { return a < b ? a : b; }
 
 template <int BITS, int HPB> struct Lay {
     static constexpr int NB = 16 * BITS;            // bytes per packed row
     static constexpr int PC = NB * 8;               // bit lanes per row
     static constexpr int GPW = kWave / NB;          // 4-token groups per wave pass
     static constexpr int TPW = 4 * GPW;             // tokens per wave pass
-    static constexpr int KT = NB * 256 * HPB * 4;   // K table bytes
-    static constexpr int SPREAD = 256 * 8;
-    static constexpr int WTAB = kNW * GPW * 16 * HPB * 4;
-    static constexpr int VSTAGE = kVSub * NB;
-    static constexpr int VNEED = SPREAD + WTAB + VSTAGE;
-    static constexpr int RED = kNW * PC * HPB * 4;
-    static constexpr int RED2 = kNW * kD * HPB * 4;
-    static constexpr int A0 = KT > VNEED ? KT : VNEED;
-    static constexpr int A1 = RED > RED2 ? RED : RED2;
-    static constexpr int REGION_A = A0 > A1 ? A0 : A1;
+    static constexpr int ESZ = HPB * 4;             // bytes per fp32 table entry / logits slot
+    static constexpr int HW = HPB >= 2 ? HPB / 2 : 1;   // 32-bit words per packed-fp16 entry
+    static constexpr int ESZH = HW * 4;             // bytes per packed-fp16 table entry
+    static constexpr int KT = NB * 256 * ESZ;       // K table bytes
+    static constexpr int SPREAD = 4 * 256 * 8;      // four spread tables
+    static constexpr int WTAB = kNW * GPW * 16 * ESZH;
+    static constexpr int VSUB = kNT * kPF / BITS;   // V tokens staged at a time
+    static constexpr int KR = kPF / BITS;           // K token rounds in flight per thread
+    static constexpr int RED = kNW * PC * ESZ;
+    static constexpr int RED2 = kNW * kD * ESZ;
     // fixed small region (floats)
     static constexpr int F_WBIT = 0;                          // NB*8*HPB
-    static constexpr int F_ZSUM = F_WBIT + NB * 8 * HPB;      // NB*HPB
-    static constexpr int F_QF = F_ZSUM + NB * HPB;            // HPB*kD
+    static constexpr int F_QF = F_WBIT + NB * 8 * HPB;        // HPB*kD
     static constexpr int F_QSZ = F_QF + HPB * kD;             // HPB*kD
-    static constexpr int F_RED = F_QSZ + HPB * kD;            // kNW*HPB*2
-    static constexpr int F_BC = F_RED + kNW * HPB * 2;        // 4*HPB broadcast slots
-    static constexpr int F_SRES = F_BC + 4 * HPB;             // kResTile*HPB
+    static constexpr int F_QRAW = F_QSZ + HPB * kD;           // HPB*kD raw 16-bit q
+    static constexpr int F_RED = F_QRAW + HPB * kD / 2;       // kNW*HPB
+    static constexpr int F_STAT = F_RED + kNW * HPB;          // 8*HPB: per-head softmax state
+    static constexpr int F_VSZ = F_STAT + 8 * HPB;            // 2*kD: value scale, zero-point
+    static constexpr int F_NIB = F_VSZ + 2 * kD;              // NB*32*HPB: nibble tables
+    static constexpr int F_SRES = F_NIB + NB * 32 * HPB;      // kResTile*HPB
     static constexpr int F_PRES = F_SRES + kResTile * HPB;    // kResTile*HPB
     static constexpr int F_END = F_PRES + kResTile * HPB;
-    static constexpr int FIXED = ((F_END * 4 + 15) / 16) * 16;
-    static constexpr int max_chunk() { return ((kLdsMax - REGION_A - FIXED) / (HPB * 4)) / 64 * 64; }
-    static constexpr int lds_bytes(int cap) { return REGION_A + FIXED + cap * HPB * 4; }
+    static constexpr int FIXED = ((F_END * 4 + 255) / 256) * 256;
+    static constexpr int region_a(int cap) {
+        return (cmax(cmax(KT, SPREAD + WTAB + cmin(VSUB, cap) * NB), cmax(RED, RED2)) + 255) / 256 * 256;
+    }
+    static constexpr int lds_bytes(int cap) { return region_a(cap) + FIXED + cap * ESZ; }
+    static constexpr int max_chunk() {
+        int best = 64;
+        for (int c = 64; c <= 16384; c += 64)
+            if (lds_bytes(c) <= kLdsMax) best = c;
+        return best;
+    }
 };
 
-__device__ __forceinline__ void wave_lds_fence() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
-// Block-wide reduction of HPB values with `op`; result broadcast to all threads.
+// Block-wide reduction of HPB values with `op`; result broadcast to all threads
+// (wave-uniform, so it can live in scalar registers).
 template <int HPB, typename Op>
 __device__ __forceinline__ void block_reduce(float* v, float* red, Op op, float identity) {
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
 #pragma unroll
     for (int h = 0; h < HPB; ++h) {
-        float x = v[h];
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) x = op(x, __shfl_xor(x, o, kWave));
+        const float x = wave_reduce(v[h], op, identity);
         if (lane == 0) red[w * HPB + h] = x;
     }
     __syncthreads();
+    static_assert(kNW <= 16, "second stage folds at most 16 wave partials");
 #pragma unroll
     for (int h = 0; h < HPB; ++h) {
-        float x = identity;
-#pragma unroll
-        for (int i = 0; i < kNW; ++i) x = op(x, red[i * HPB + h]);
-        v[h] = x;
+        float x = (lane < kNW) ? red[lane * HPB + h] : identity;
+        x = row_reduce(x, op, identity);   // lanes 0..15 hold the partials
+        v[h] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, x)));
     }
     __syncthreads();
 }
-
-struct OpMin { __device__ float operator()(float a, float b) const { return fminf(a, b); } };
-struct OpMax { __device__ float operator()(float a, float b) const { return fmaxf(a, b); } };
-struct OpSum { __device__ float operator()(float a, float b) const { return a + b; } };
 
 // Unit decomposition of a 1-D grid.  Consecutive work ids share packed codes
 // (head groups of one kv-head), so when the grid is a multiple of the 8 XCDs
@@ -129,21 +139,51 @@ __device__ __forceinline__ int virtual_block_id() {
     return l;
 }
 
+// Two-element dot product with fp32 accumulation on raw 16-bit pairs.
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+template <typename DT> __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c);
+template <> __device__ __forceinline__ float dot2<BF16>(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c, false);
+}
+template <> __device__ __forceinline__ float dot2<FP16>(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, a), __builtin_bit_cast(f16x2_t, b), c, false);
+}
+
+template <int N> struct alignas(N * 4) Words { uint32_t w[N]; };
+
+// x + (x of lane ^ 16) and x + (x of lane ^ 32) with the row / half-wave swap
+// instructions: a copy is swapped against the original, then the pair is added.
+__device__ __forceinline__ float add_lane_xor16(float x) {
+    uint32_t a = __builtin_bit_cast(uint32_t, x), b;
+    asm volatile("v_mov_b32 %1, %0\n\ts_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "=&v"(b));
+    return __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b);
+}
+__device__ __forceinline__ float add_lane_xor32(float x) {
+    uint32_t a = __builtin_bit_cast(uint32_t, x), b;
+    asm volatile("v_mov_b32 %1, %0\n\ts_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "=&v"(b));
+    return __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b);
+}
+
+__device__ __forceinline__ uint32_t pack_f16(float a, float b) {
+    f16x2_t h = {static_cast<_Float16>(a), static_cast<_Float16>(b)};   // round to nearest even
+    return __builtin_bit_cast(uint32_t, h);
+}
+
 template <int BITS, int HPB, typename DT, bool MINMAX_ONLY>
 __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
     using L = Lay<BITS, HPB>;
     using V = Vec<HPB>;
     constexpr int NB = L::NB;
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    extern __shared__ __attribute__((aligned(256))) unsigned char smem[];
+    const int reg_a = L::region_a(g.cap);
     unsigned char* regA = smem;
-    float* fx = reinterpret_cast<float*>(smem + L::REGION_A);
-    V* logits = reinterpret_cast<V*>(smem + L::REGION_A + L::FIXED);
+    float* fx = reinterpret_cast<float*>(smem + reg_a);
+    V* logits = reinterpret_cast<V*>(smem + reg_a + L::FIXED);
     float* wbit = fx + L::F_WBIT;
-    float* zsum = fx + L::F_ZSUM;
     float* qf = fx + L::F_QF;
     float* qsz = fx + L::F_QSZ;
     float* red = fx + L::F_RED;
-    float* bc = fx + L::F_BC;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -163,16 +203,80 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
     const bool do_res = !MINMAX_ONLY && g.R > 0 && (g.nsplit == 1 || split == g.nsplit);
     const int t0 = img_unit ? split * g.chunk : 0;
     const int n = img_unit ? min(g.T, t0 + g.chunk) - t0 : 0;
+    const int npad = (n + L::TPW - 1) / L::TPW * L::TPW;
     const float inv_sqrt_d = 0.08838834764831845f;  // 1/sqrt(128)
 
-    // ---- phase 0: q, per-bit weights, zero-point sums ------------------------
+    // ---- entry: put the unit's global loads in flight.  The vector-memory counter is
+    // in order, so the few elements phase 0 needs are requested first and the bulk
+    // streams (packed K, packed V, residual tile) behind them.
+    // Loads are unconditional with clamped (always valid) addresses: no divergent
+    // control flow around them, so the compiler can wait on exactly the counter value
+    // each consumer needs.
+    // A unit without packed tokens or without residual rows aims the unused streams
+    // at q (always mapped, at least 256 bytes) and never looks at what comes back.
+    const bool has_img = n > 0;
+    uint32_t q_raw, s_raw, z_raw;
+    {
+        const int h = min(tid / kD, HPB - 1), d = tid % kD;
+        const uint16_t* qp = static_cast<const uint16_t*>(g.q) + (static_cast<int64_t>(b) * g.Hq + hq0) * kD;
+        q_raw = qp[h * kD + d];
+        const bool vstat = tid >= kNT - kD;   // the last kD threads fetch the value statistics
+        const uint16_t* sp = has_img ? static_cast<const uint16_t*>(vstat ? g.vs : g.ks) + bh * kD : qp;
+        const uint16_t* zp = has_img ? static_cast<const uint16_t*>(vstat ? g.vz : g.kz) + bh * kD : qp;
+        s_raw = sp[d];
+        z_raw = zp[d];
+    }
+    const uint4* ckp = has_img ? reinterpret_cast<const uint4*>(g.ck + (bh * g.T + t0) * NB)
+                               : static_cast<const uint4*>(g.q);
+    const uint4* cvp = has_img ? reinterpret_cast<const uint4*>(g.cv + (bh * g.T + t0) * NB)
+                               : static_cast<const uint4*>(g.q);
+    const U4* cvp4 = reinterpret_cast<const U4*>(cvp);
+    const int last_u = has_img ? n * NB / 16 - 1 : 0;   // last valid 16-byte unit of either stream
+    uint4 kc[L::KR][BITS];
+#pragma unroll
+    for (int r = 0; r < L::KR; ++r) {
+#pragma unroll
+        for (int i = 0; i < BITS; ++i) kc[r][i] = ckp[min((tid + r * kNT) * BITS + i, last_u)];
+    }
+    // residual tile: K slice (row = tid/8, 16 elements) and V slices (two rows, 8 elements)
+    const int l8 = tid & 7, krow = tid >> 3;
+    // residual V: lane = (8-element slice ds, row slot): the slot's two low bits sit in the
+    // two low lane bits so the final fold over slots is a quad permute
+    const int ds = (tid >> 2) & 15, rslot = (tid & 3) | ((tid >> 6) << 2);
+    const uint16_t* kb = do_res ? static_cast<const uint16_t*>(g.kres) + b * g.rs_b + hkv * g.rs_h
+                                : static_cast<const uint16_t*>(g.q);
+    const uint16_t* vbp = do_res ? static_cast<const uint16_t*>(g.vres) + b * g.rs_b + hkv * g.rs_h
+                                 : static_cast<const uint16_t*>(g.q);
+    const int last_r = do_res ? g.R - 1 : 0;
+    const int64_t rs_r = do_res ? g.rs_r : 0;
+    uint4 rk[2], rv[2];
+    auto load_res_k = [&](int r0, uint4* k2) {   // rows past R re-read row R-1 (their logit is masked)
+        const uint16_t* kp = kb + min(r0 + krow, last_r) * rs_r;
+        k2[0] = *reinterpret_cast<const uint4*>(kp + l8 * 8);
+        k2[1] = *reinterpret_cast<const uint4*>(kp + 64 + l8 * 8);
+    };
+    auto load_res_v = [&](int r0, uint4* v2) {   // rows past R re-read row R-1 (their weight is 0)
+#pragma unroll
+        for (int rep = 0; rep < 2; ++rep) {
+            const int r2 = min(r0 + rslot + rep * (kResTile / 2), last_r);
+            v2[rep] = *reinterpret_cast<const uint4*>(vbp + r2 * rs_r + ds * 8);
+        }
+    };
+    if constexpr (!MINMAX_ONLY) {
+        load_res_k(0, rk);
+        load_res_v(0, rv);
+    }
+
+    // ---- phase 0: q, per-bit weights ---------------------------------------------------
     if (tid < HPB * kD) {
         const int h = tid / kD, d = tid % kD;
-        const float qv = load_elem<DT>(g.q, (static_cast<int64_t>(b) * g.Hq + hq0 + h) * kD + d) * inv_sqrt_d;
+        const float qraw = Cvt<DT>::to_float(q_raw);
+        reinterpret_cast<uint16_t*>(fx + L::F_QRAW)[h * kD + d] = static_cast<uint16_t>(q_raw);
+        const float qv = qraw * inv_sqrt_d;
         qf[h * kD + d] = qv;
         if (n > 0) {
-            const float s = load_elem<DT>(g.ks, bh * kD + d);
-            const float z = load_elem<DT>(g.kz, bh * kD + d);
+            const float s = Cvt<DT>::to_float(s_raw);
+            const float z = Cvt<DT>::to_float(z_raw);
             const float qs = qv * s;
             qsz[h * kD + d] = qs * z;
             if constexpr (BITS == 1) {
@@ -184,101 +288,198 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
             }
         }
     }
+    if (n > 0 && tid >= kNT - kD && tid >= HPB * kD) {
+        const int d = tid - (kNT - kD);
+        fx[L::F_VSZ + d] = Cvt<DT>::to_float(s_raw);
+        fx[L::F_VSZ + kD + d] = Cvt<DT>::to_float(z_raw);
+    }
     __syncthreads();
 
     float mn[HPB], mx[HPB];
 #pragma unroll
     for (int h = 0; h < HPB; ++h) { mn[h] = INFINITY; mx[h] = -INFINITY; }
+    U4 vc[kPF];   // first block of packed V rows, requested as the packed K registers free up
 
     if (n > 0) {
-        if (tid < NB * HPB) {
-            const int j = tid / HPB, h = tid % HPB;
+        // ---- phase 1: byte table = high-nibble table + low-nibble table ----------------
+        // nibble tables: entry (j, half, v) = sum of the per-bit weights v selects; the
+        // zero-point sum of the byte position is folded into the high half.
+        V* nib = reinterpret_cast<V*>(fx + L::F_NIB);   // [half*16 + value][byte position]
+        V* ktab = reinterpret_cast<V*>(regA);           // [byte value][byte position]
+        for (int e = tid; e < NB * 32; e += kNT) {
+            const int j = e % NB, half = (e / NB) >> 4, v = (e / NB) & 15;
+            const V* wb = reinterpret_cast<const V*>(wbit) + j * 8 + half * 4;
             constexpr int cpb = 8 / BITS;
-            float s = 0.f;
-#pragma unroll
-            for (int i = 0; i < cpb; ++i) s += qsz[h * kD + j * cpb + i];
-            zsum[j * HPB + h] = s;
-        }
-        __syncthreads();
-
-        // ---- phase 1: byte table.  Thread = (byte position, high nibble);
-        // the 16 low-nibble values are walked in Gray-code order so each entry
-        // costs one add per head.
-        V* ktab = reinterpret_cast<V*>(regA);
-        for (int pr = tid; pr < NB * 16; pr += kNT) {
-            const int j = pr >> 4, vhi = pr & 15;
-            const V* wb = reinterpret_cast<const V*>(wbit) + j * 8;
             V acc;
-            const V zs = reinterpret_cast<const V*>(zsum)[j];
 #pragma unroll
-            for (int h = 0; h < HPB; ++h) acc.v[h] = -zs.v[h];
+            for (int h = 0; h < HPB; ++h) {
+                float zs = 0.f;
+                if (half) {
+#pragma unroll
+                    for (int i = 0; i < cpb; ++i) zs += qsz[h * kD + j * cpb + i];
+                }
+                acc.v[h] = -zs;
+            }
 #pragma unroll
             for (int bt = 0; bt < 4; ++bt) {
-                const V wv4 = wb[4 + bt];
-                const float f = static_cast<float>((vhi >> bt) & 1);
+                const V w4 = wb[bt];
+                const float f = static_cast<float>((v >> bt) & 1);
 #pragma unroll
-                for (int h = 0; h < HPB; ++h) acc.v[h] += f * wv4.v[h];
+                for (int h = 0; h < HPB; ++h) acc.v[h] += f * w4.v[h];
             }
-            V wlo[4];
+            nib[e] = acc;
+        }
+        __syncthreads();
+        for (int e = tid; e < NB * 256; e += kNT) {
+            const int j = e % NB, v = e / NB;
+            const V hi = nib[(16 + (v >> 4)) * NB + j];
+            const V lo = nib[(v & 15) * NB + j];
+            V o;
 #pragma unroll
-            for (int bt = 0; bt < 4; ++bt) wlo[bt] = wb[bt];
-            V* dst = ktab + j * 256 + vhi * 16;
-            dst[0] = acc;
-#pragma unroll
-            for (int k = 1; k < 16; ++k) {
-                const int gray = k ^ (k >> 1);
-                const int bt = __builtin_ctz(k);
-                const bool set = (gray >> bt) & 1;
-#pragma unroll
-                for (int h = 0; h < HPB; ++h) acc.v[h] = set ? acc.v[h] + wlo[bt].v[h] : acc.v[h] - wlo[bt].v[h];
-                dst[gray] = acc;
-            }
+            for (int h = 0; h < HPB; ++h) o.v[h] = hi.v[h] + lo.v[h];
+            ktab[e] = o;
         }
         __syncthreads();
 
-        // ---- phase 2: logits of the chunk ------------------------------------
-        const uint8_t* ckb = g.ck + (bh * g.T + t0) * NB;
-        for (int tt = tid; tt < n; tt += kNT) {
-            const uint4* cp = reinterpret_cast<const uint4*>(ckb + static_cast<int64_t>(tt) * NB);
-            uint32_t wds[4 * BITS];
+        // ---- phase 2: logits of the chunk ------------------------------------------------
+        // Lane l walks the byte positions in the order k ^ (l mod NB): in every step the
+        // lanes that the LDS serves together read NB distinct positions of the
+        // position-fastest table, i.e. distinct banks whatever the byte values are.  The
+        // row is permuted by the same XOR once, so step k finds its byte at a fixed place.
+        // The NB terms are added as a balanced binary tree over k; an XOR of the leaf index
+        // only swaps the two children of some tree levels, so every lane gets bit-identical
+        // logits for identical rows.
+        constexpr int NW32 = NB / 4;
+        const int skew = lane % NB;
+        // byte i of a word <- byte i ^ (skew & 3)
+        const uint32_t bsel = (0x03020100u ^ (0x01010101u * (skew & 3)));
+        uint32_t pofs[NB];   // byte offset of position k ^ skew inside a table row
 #pragma unroll
-            for (int i = 0; i < BITS; ++i) {
-                const uint4 c = cp[i];
-                wds[4 * i + 0] = c.x; wds[4 * i + 1] = c.y; wds[4 * i + 2] = c.z; wds[4 * i + 3] = c.w;
+        for (int k = 0; k < NB; ++k) pofs[k] = (k ^ skew) * L::ESZ;
+        const unsigned char* ktab_b = regA;
+        auto token_logits = [&](int tt, const uint4* c) {
+            if (tt < n) {
+                uint32_t w[NW32];
+#pragma unroll
+                for (int i = 0; i < BITS; ++i) {
+                    w[4 * i + 0] = c[i].x; w[4 * i + 1] = c[i].y;
+                    w[4 * i + 2] = c[i].z; w[4 * i + 3] = c[i].w;
+                }
+#pragma unroll
+                for (int st = 0; (1 << st) < NW32; ++st) {   // word i <- word i ^ (skew / 4)
+                    const bool on = ((skew >> 2) >> st) & 1;
+                    uint32_t t[NW32];
+#pragma unroll
+                    for (int i = 0; i < NW32; ++i) t[i] = w[i ^ (1 << st)];
+#pragma unroll
+                    for (int i = 0; i < NW32; ++i) w[i] = on ? t[i] : w[i];
+                }
+                uint32_t wds[NW32];
+#pragma unroll
+                for (int i = 0; i < NW32; ++i) wds[i] = __builtin_amdgcn_perm(w[i], w[i], bsel);
+                // balanced-tree sum with a small stack of partial sums (level l holds 2^l terms)
+                V part[6];
+#pragma unroll
+                for (int k = 0; k < NB; ++k) {
+                    const uint32_t byte = (wds[k >> 2] >> (8 * (k & 3))) & 0xffu;
+                    V cur = *reinterpret_cast<const V*>(ktab_b + byte * (NB * L::ESZ) + pofs[k]);
+#pragma unroll
+                    for (int l = 0; l < 6; ++l) {
+                        if ((k >> l) & 1) {
+#pragma unroll
+                            for (int h = 0; h < HPB; ++h) cur.v[h] += part[l].v[h];
+                        } else {
+                            part[l] = cur;
+                            break;
+                        }
+                    }
+                    if (k == NB - 1) part[5] = cur;
+                    // keep at most 8 look-ups in flight: bounds the registers this loop needs
+                    if ((k & 7) == 7) __builtin_amdgcn_sched_barrier(0);
+                }
+                const V acc = part[5];
+                if constexpr (!MINMAX_ONLY) logits[tt] = acc;
+#pragma unroll
+                for (int h = 0; h < HPB; ++h) { mn[h] = fminf(mn[h], acc.v[h]); mx[h] = fmaxf(mx[h], acc.v[h]); }
             }
-            V acc;
-#pragma unroll
-            for (int h = 0; h < HPB; ++h) acc.v[h] = 0.f;
-#pragma unroll
-            for (int j = 0; j < NB; ++j) {
-                const uint32_t byte = (wds[j >> 2] >> (8 * (j & 3))) & 0xffu;
-                const V e = ktab[j * 256 + byte];
-#pragma unroll
-                for (int h = 0; h < HPB; ++h) acc.v[h] += e.v[h];
-            }
-            if constexpr (!MINMAX_ONLY) logits[tt] = acc;
-#pragma unroll
-            for (int h = 0; h < HPB; ++h) { mn[h] = fminf(mn[h], acc.v[h]); mx[h] = fmaxf(mx[h], acc.v[h]); }
+        };
+        // first batch: rows already in registers; each consumed round frees registers
+        // that take the first block of packed V rows
+        // (written out round by round with constant indices so vc stays in registers)
+#define CQ_K_ROUND(R)                                                                         \
+        if constexpr (L::KR > (R)) {                                                          \
+            token_logits(tid + (R) * kNT, kc[(R)]);                                           \
+            if constexpr (!MINMAX_ONLY) {                                                     \
+                vc[(R) * BITS] = cvp4[min(tid + ((R) * BITS) * kNT, last_u)];                 \
+                if constexpr (BITS == 2)                                                      \
+                    vc[(R) * BITS + 1] = cvp4[min(tid + ((R) * BITS + 1) * kNT, last_u)];     \
+            }                                                                                 \
         }
+        CQ_K_ROUND(0)
+        CQ_K_ROUND(1)
+        CQ_K_ROUND(2)
+        CQ_K_ROUND(3)
+#undef CQ_K_ROUND
+        static_assert(L::KR <= 4, "rounds are written out up to 4");
+        for (int tb = kNT * L::KR; tb < n; tb += kNT * L::KR) {
+#pragma unroll
+            for (int r = 0; r < L::KR; ++r) {
+                const int tt = min(tb + tid + r * kNT, n - 1);
+#pragma unroll
+                for (int i = 0; i < BITS; ++i) kc[r][i] = ckp[static_cast<int64_t>(tt) * BITS + i];
+            }
+#pragma unroll
+            for (int r = 0; r < L::KR; ++r) token_logits(tb + tid + r * kNT, kc[r]);
+        }
+    }
+    if (n > 0) {
         block_reduce<HPB>(mn, red, OpMin(), INFINITY);
         block_reduce<HPB>(mx, red, OpMax(), -INFINITY);
     }
 
     if constexpr (MINMAX_ONLY) {
-        if (n > 0 && tid < HPB) {
-            float* o = g.mm + ((static_cast<int64_t>(b) * g.Hq + hq0 + tid) * g.nsplit + split) * 2;
-            o[0] = mn[tid];
-            o[1] = mx[tid];
+#pragma unroll
+        for (int h = 0; h < HPB; ++h) {
+            if (n > 0 && tid == h) {
+                float* o = g.mm + ((static_cast<int64_t>(b) * g.Hq + hq0 + h) * g.nsplit + split) * 2;
+                o[0] = mn[h];
+                o[1] = mx[h];
+            }
         }
         return;
     } else {
-        // ---- phase 3: calibration + exp -------------------------------------------
         float m_img[HPB], l_img[HPB];
 #pragma unroll
         for (int h = 0; h < HPB; ++h) { m_img[h] = -INFINITY; l_img[h] = 0.f; }
         float o_img = 0.f;  // thread (h, d) = (tid / kD, tid % kD) for tid < HPB*kD
 
         if (n > 0) {
+            // the K table is dead: stage the first block of packed V rows and the
+            // spread tables in its place (ordered by the barriers of block_reduce)
+            uint2* spread = reinterpret_cast<uint2*>(regA);
+            unsigned char* vst = regA + L::SPREAD + L::WTAB;
+            {
+                const int c = tid & 255, pos = tid >> 8;   // kNT == 4 * 256
+                uint32_t lo = 0, hi = 0;
+#pragma unroll
+                for (int m = 0; m < 4; ++m) {
+                    lo |= ((c >> (7 - m)) & 1u) << (8 * m);
+                    hi |= ((c >> (3 - m)) & 1u) << (8 * m);
+                }
+                constexpr int esh = L::ESZH == 8 ? 3 : 2;
+                spread[pos * 256 + c] = make_uint2(lo << (esh + pos), hi << (esh + pos));
+            }
+
+            {
+                const int vn0 = min(L::VSUB, npad);
+#pragma unroll
+                for (int r = 0; r < kPF; ++r) {
+                    const int u = tid + r * kNT;
+                    if (u < vn0 * NB / 16) reinterpret_cast<U4*>(vst)[u] = vc[r];
+                }
+            }
+
+            // ---- phase 3: calibration + exp ---------------------------------------------
             if (g.nsplit > 1) {
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) {
@@ -300,7 +501,6 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                     slope[h] = 1.0f;
                 }
             }
-            const int npad = (n + L::TPW - 1) / L::TPW * L::TPW;
             if (g.mask) {
                 const float* mk = g.mask + b * g.mask_sb + g.S + t0;
                 float lm[HPB];
@@ -326,108 +526,120 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
             float ls[HPB];
 #pragma unroll
             for (int h = 0; h < HPB; ++h) ls[h] = 0.f;
+            using HWv = Words<L::HW>;
             for (int tt = tid; tt < npad; tt += kNT) {
-                V w;
+                float e[4] = {0.f, 0.f, 0.f, 0.f};
                 if (tt < n) {
-                    w = logits[tt];
+                    const V w = logits[tt];
 #pragma unroll
                     for (int h = 0; h < HPB; ++h) {
                         const float x = (w.v[h] - mn[h]) * slope[h] + tmin[h];
-                        const float e = (m_img[h] == -INFINITY) ? 0.f : __expf(x - m_img[h]);
-                        w.v[h] = e;
-                        ls[h] += e;
+                        e[h] = (m_img[h] == -INFINITY) ? 0.f : __expf(x - m_img[h]);
+                        ls[h] += e[h];
                     }
-                } else {
-#pragma unroll
-                    for (int h = 0; h < HPB; ++h) w.v[h] = 0.f;
                 }
-                logits[tt] = w;
+                // e as packed fp16 in the first bytes of the token's slot (read by the V tables)
+                HWv hw;
+                hw.w[0] = pack_f16(e[0], e[1]);
+                if constexpr (L::HW == 2) hw.w[1] = pack_f16(e[2], e[3]);
+                *reinterpret_cast<HWv*>(&logits[tt]) = hw;
             }
-            block_reduce<HPB>(ls, red, OpSum(), 0.f);
+            block_reduce<HPB>(ls, red, OpSum(), 0.f);   // its barriers also publish e, spread, vst
 #pragma unroll
             for (int h = 0; h < HPB; ++h) l_img[h] = ls[h];
 
-            // ---- phase 4: packed V ----------------------------------------------------
-            uint2* spread = reinterpret_cast<uint2*>(regA);
-            V* wtab = reinterpret_cast<V*>(regA + L::SPREAD) + wv * (L::GPW * 16);
-            unsigned char* vst = regA + L::SPREAD + L::WTAB;
-            if (tid < 256) {
-                uint32_t lo = 0, hi = 0;
-#pragma unroll
-                for (int m = 0; m < 4; ++m) {
-                    lo |= ((tid >> (7 - m)) & 1u) << (8 * m);
-                    hi |= ((tid >> (3 - m)) & 1u) << (8 * m);
-                }
-                spread[tid] = make_uint2(lo, hi);
-            }
+            // ---- phase 4: packed V ----------------------------------------------------------
+            unsigned char* wtab = regA + L::SPREAD + wv * (L::GPW * 16 * L::ESZH);
             const int j = lane % NB, gs = lane / NB;
             const int bg = lane >> 4, be = lane & 15;   // table build: group, entry
-            float bsel[4];
+            f16x2_t bsel[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) bsel[i] = static_cast<float>((be >> i) & 1);
-            V acc[8];
+            for (int i = 0; i < 4; ++i) {
+                const _Float16 f = static_cast<_Float16>(static_cast<float>((be >> i) & 1));
+                bsel[i] = f16x2_t{f, f};
+            }
+            float acc[8][HPB];
 #pragma unroll
             for (int m = 0; m < 8; ++m)
 #pragma unroll
-                for (int h = 0; h < HPB; ++h) acc[m].v[h] = 0.f;
-            const uint8_t* cvb = g.cv + (bh * g.T + t0) * NB;
+                for (int h = 0; h < HPB; ++h) acc[m][h] = 0.f;
+            const float one = g.one;
 
-            for (int vs0 = 0; vs0 < npad; vs0 += kVSub) {
-                const int vn = min(kVSub, npad - vs0);
-                __syncthreads();  // previous sub-chunk consumed (and spread written)
-                for (int u = tid; u < vn * NB / 16; u += kNT) {
-                    const int tok = vs0 + u * 16 / NB;
-                    uint4 c = make_uint4(0, 0, 0, 0);
-                    if (tok < n) c = reinterpret_cast<const uint4*>(cvb + static_cast<int64_t>(vs0) * NB)[u];
-                    reinterpret_cast<uint4*>(vst)[u] = c;
+            for (int vs0 = 0; vs0 < npad; vs0 += L::VSUB) {
+                const int vn = min(L::VSUB, npad - vs0);
+                if (vs0 > 0) {
+                    __syncthreads();  // previous block consumed
+                    for (int u = tid; u < vn * NB / 16; u += kNT) {
+                        const int tok = vs0 + u * 16 / NB;
+                        uint4 c = make_uint4(0, 0, 0, 0);
+                        if (tok < n) c = cvp[static_cast<int64_t>(vs0) * NB / 16 + u];
+                        reinterpret_cast<uint4*>(vst)[u] = c;
+                    }
+                    __syncthreads();
                 }
-                __syncthreads();
                 for (int u = wv; u * L::TPW < vn; u += kNW) {
-                    const int tl = u * L::TPW;        // token offset inside the sub-chunk
+                    const int tl = u * L::TPW;        // token offset inside the block
                     if (bg < L::GPW) {
-                        V val;
+                        // entry `be` of group `bg`: fp16 sum of the e values its bits select
+                        f16x2_t val[L::HW];
 #pragma unroll
-                        for (int h = 0; h < HPB; ++h) val.v[h] = 0.f;
+                        for (int k = 0; k < L::HW; ++k) val[k] = f16x2_t{0, 0};
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
-                            const V e = logits[vs0 + tl + 4 * bg + i];
+                            const HWv e = *reinterpret_cast<const HWv*>(&logits[vs0 + tl + 4 * bg + i]);
 #pragma unroll
-                            for (int h = 0; h < HPB; ++h) val.v[h] += bsel[i] * e.v[h];
+                            for (int k = 0; k < L::HW; ++k) val[k] += __builtin_bit_cast(f16x2_t, e.w[k]) * bsel[i];
                         }
-                        wtab[bg * 16 + be] = val;
+                        HWv o;
+#pragma unroll
+                        for (int k = 0; k < L::HW; ++k) o.w[k] = __builtin_bit_cast(uint32_t, val[k]);
+                        reinterpret_cast<HWv*>(wtab)[bg * 16 + be] = o;
                     }
-                    wave_lds_fence();
                     uint32_t xlo = 0, xhi = 0;
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const uint32_t c = vst[(tl + 4 * gs + i) * NB + j];
-                        const uint2 sp = spread[c];
-                        xlo |= sp.x << i;
-                        xhi |= sp.y << i;
+                        const uint2 sp = spread[i * 256 + c];
+                        xlo |= sp.x;
+                        xhi |= sp.y;
                     }
-                    const V* tb = wtab + gs * 16;
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                    const unsigned char* tbp = wtab + gs * (16 * L::ESZH);
 #pragma unroll
                     for (int m = 0; m < 8; ++m) {
                         const uint32_t x = m < 4 ? xlo : xhi;
-                        const V e = tb[(x >> (8 * (m & 3))) & 15u];
+                        const HWv e = *reinterpret_cast<const HWv*>(tbp + ((x >> (8 * (m & 3))) & 0xffu));
 #pragma unroll
-                        for (int h = 0; h < HPB; ++h) acc[m].v[h] += e.v[h];
+                        for (int h = 0; h < HPB; ++h) {
+                            const f16x2_t pr = __builtin_bit_cast(f16x2_t, e.w[h >> 1]);
+                            const _Float16 hv = (h & 1) ? pr.y : pr.x;
+                            acc[m][h] = __builtin_fmaf(static_cast<float>(hv), one, acc[m][h]);
+                        }
                     }
-                    wave_lds_fence();
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
                 }
             }
             // fold the group slots of the wave, then the waves
 #pragma unroll
-            for (int o = NB; o < kWave; o <<= 1)
+            for (int m = 0; m < 8; ++m)
 #pragma unroll
-                for (int m = 0; m < 8; ++m)
-#pragma unroll
-                    for (int h = 0; h < HPB; ++h) acc[m].v[h] += __shfl_xor(acc[m].v[h], o, kWave);
+                for (int h = 0; h < HPB; ++h) {
+                    if constexpr (L::GPW == 4) acc[m][h] = add_lane_xor16(acc[m][h]);
+                    acc[m][h] = add_lane_xor32(acc[m][h]);
+                }
             __syncthreads();
             V* redv = reinterpret_cast<V*>(regA);  // [wave][PC]
             if (gs == 0) {
 #pragma unroll
-                for (int m = 0; m < 8; ++m) redv[wv * L::PC + j * 8 + m] = acc[m];
+                for (int m = 0; m < 8; ++m) {
+                    V a4;
+#pragma unroll
+                    for (int h = 0; h < HPB; ++h) a4.v[h] = acc[m][h];
+                    redv[wv * L::PC + j * 8 + m] = a4;
+                }
             }
             __syncthreads();
             if (tid < HPB * kD) {
@@ -441,9 +653,8 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                     for (int w = 0; w < kNW; ++w)
                         a += 2.0f * redv[w * L::PC + 2 * d].v[h] + redv[w * L::PC + 2 * d + 1].v[h];
                 }
-                const float s = load_elem<DT>(g.vs, bh * kD + d);
-                const float z = load_elem<DT>(g.vz, bh * kD + d);
-                // pick this thread's head out of the per-head sums
+                const float s = fx[L::F_VSZ + d];
+                const float z = fx[L::F_VSZ + kD + d];
                 float lh = l_img[0];
 #pragma unroll
                 for (int k = 1; k < HPB; ++k) lh = (h == k) ? l_img[k] : lh;
@@ -452,112 +663,95 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
             __syncthreads();
         }
 
-        // ---- phase 5: full-precision residual rows, online softmax ----------------
-        float m_res[HPB], l_res[HPB];
+        // ---- phase 5: full-precision residual rows, online softmax ----------------------
+        float* stat = fx + L::F_STAT;   // [alpha | m_res | l_res | m_img | l_img][HPB]
 #pragma unroll
-        for (int h = 0; h < HPB; ++h) { m_res[h] = -INFINITY; l_res[h] = 0.f; }
+        for (int h = 0; h < HPB; ++h) {
+            if (tid == h) {
+                stat[HPB + h] = -INFINITY;
+                stat[2 * HPB + h] = 0.f;
+                stat[3 * HPB + h] = m_img[h];
+                stat[4 * HPB + h] = l_img[h];
+            }
+        }
         float o_res = 0.f;
         if (do_res) {
+            float m_run = -INFINITY, l_run = 0.f;
             float* sres = fx + L::F_SRES;
             float* pres = fx + L::F_PRES;
-            const int l8 = tid & 7, row = tid >> 3;
-            const int ds = tid & 15, rslot = tid >> 4;
-            float qa[HPB][16];
-#pragma unroll
-            for (int h = 0; h < HPB; ++h)
-#pragma unroll
-                for (int k = 0; k < 8; ++k) {
-                    qa[h][k] = qf[h * kD + l8 * 8 + k];
-                    qa[h][8 + k] = qf[h * kD + 64 + l8 * 8 + k];
-                }
+            // raw 16-bit q, [head][kD], read per head as two 16-byte LDS loads
+            const uint4* q128 = reinterpret_cast<const uint4*>(fx + L::F_QRAW);
             float accv[8][HPB];
 #pragma unroll
             for (int k = 0; k < 8; ++k)
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) accv[k][h] = 0.f;
-            const uint16_t* kb = static_cast<const uint16_t*>(g.kres) + b * g.rs_b + hkv * g.rs_h;
-            const uint16_t* vbp = static_cast<const uint16_t*>(g.vres) + b * g.rs_b + hkv * g.rs_h;
             const float* mk = g.mask ? g.mask + b * g.mask_sb : nullptr;
 
             for (int r0 = 0; r0 < g.R; r0 += kResTile) {
-                const int r = r0 + row;
+                const bool more = r0 + kResTile < g.R;
+                const int r = r0 + krow;
                 float dot[HPB];
 #pragma unroll
-                for (int h = 0; h < HPB; ++h) dot[h] = 0.f;
-                if (r < g.R) {
-                    const uint16_t* kp = kb + r * g.rs_r;
-                    const uint4 v0 = *reinterpret_cast<const uint4*>(kp + l8 * 8);
-                    const uint4 v1 = *reinterpret_cast<const uint4*>(kp + 64 + l8 * 8);
-                    float f[16];
-                    unpack8<DT>(v0, f);
-                    unpack8<DT>(v1, f + 8);
-#pragma unroll
-                    for (int h = 0; h < HPB; ++h)
-#pragma unroll
-                        for (int k = 0; k < 16; ++k) dot[h] += qa[h][k] * f[k];
-                }
-#pragma unroll
                 for (int h = 0; h < HPB; ++h) {
-                    dot[h] += __shfl_xor(dot[h], 1, kWave);
-                    dot[h] += __shfl_xor(dot[h], 2, kWave);
-                    dot[h] += __shfl_xor(dot[h], 4, kWave);
+                    const uint4 qa = q128[h * (kD / 8) + l8];
+                    const uint4 qb = q128[h * (kD / 8) + 8 + l8];
+                    float a = 0.f;
+                    a = dot2<DT>(qa.x, rk[0].x, a); a = dot2<DT>(qa.y, rk[0].y, a);
+                    a = dot2<DT>(qa.z, rk[0].z, a); a = dot2<DT>(qa.w, rk[0].w, a);
+                    a = dot2<DT>(qb.x, rk[1].x, a); a = dot2<DT>(qb.y, rk[1].y, a);
+                    a = dot2<DT>(qb.z, rk[1].z, a); a = dot2<DT>(qb.w, rk[1].w, a);
+                    dot[h] = oct_reduce(a, OpSum(), 0.f) * inv_sqrt_d;
                 }
+                if (more) load_res_k(r0 + kResTile, rk);   // next tile's K slice, in place
                 if (l8 == 0) {
                     float mv = 0.f;
                     if (mk && r < g.R) mv = mk[r < g.S ? r : g.T + r];
 #pragma unroll
-                    for (int h = 0; h < HPB; ++h) sres[row * HPB + h] = (r < g.R) ? dot[h] + mv : -INFINITY;
+                    for (int h = 0; h < HPB; ++h) sres[krow * HPB + h] = (r < g.R) ? dot[h] + mv : -INFINITY;
+                }
+                __syncthreads();
+                if (wv < HPB) {   // wave h keeps the running softmax state of head h
+                    const int h = wv;
+                    const float s0 = sres[lane * HPB + h];
+                    const float s1 = sres[(lane + 64) * HPB + h];
+                    const float mnew = fmaxf(m_run, wave_max(fmaxf(s0, s1)));
+                    const bool dead = (mnew == -INFINITY);
+                    const float p0 = dead ? 0.f : __expf(s0 - mnew);
+                    const float p1 = dead ? 0.f : __expf(s1 - mnew);
+                    const float al = dead ? 1.0f : __expf(m_run - mnew);
+                    l_run = l_run * al + wave_sum(p0 + p1);
+                    m_run = mnew;
+                    pres[lane * HPB + h] = p0;
+                    pres[(lane + 64) * HPB + h] = p1;
+                    if (lane == 0) { stat[h] = al; stat[HPB + h] = m_run; stat[2 * HPB + h] = l_run; }
                 }
                 __syncthreads();
                 float alpha[HPB];
 #pragma unroll
-                for (int h = 0; h < HPB; ++h) {
-                    const float s = sres[lane * HPB + h];
-                    const float mt = wave_max(s);
-                    const float mnew = fmaxf(m_res[h], mt);
-                    float p = 0.f;
-                    alpha[h] = 1.0f;
-                    if (mnew != -INFINITY) {
-                        p = __expf(s - mnew);
-                        alpha[h] = __expf(m_res[h] - mnew);
-                    }
-                    const float lt = wave_sum(p);
-                    l_res[h] = l_res[h] * alpha[h] + lt;
-                    m_res[h] = mnew;
-                    if (wv == 0) pres[lane * HPB + h] = p;
+                for (int h = 0; h < HPB; ++h) alpha[h] = stat[h];
+#pragma unroll
+                for (int rep = 0; rep < 2; ++rep) {
+                    const int rr = rslot + rep * (kResTile / 2);
+                    float f[8];
+                    unpack8<DT>(rv[rep], f);
+                    const V p = reinterpret_cast<const V*>(pres)[rr];   // 0 for rows past R
+#pragma unroll
+                    for (int k = 0; k < 8; ++k)
+#pragma unroll
+                        for (int h = 0; h < HPB; ++h)
+                            accv[k][h] = (rep == 0 ? accv[k][h] * alpha[h] : accv[k][h]) + p.v[h] * f[k];
                 }
-                __syncthreads();
-#pragma unroll
-                for (int k = 0; k < 8; ++k)
-#pragma unroll
-                    for (int h = 0; h < HPB; ++h) accv[k][h] *= alpha[h];
-#pragma unroll
-                for (int rep = 0; rep < kResTile / (kNT / 16); ++rep) {
-                    const int rr = rslot + rep * (kNT / 16);
-                    const int r2 = r0 + rr;
-                    if (r2 < g.R) {
-                        const uint4 vv = *reinterpret_cast<const uint4*>(vbp + r2 * g.rs_r + ds * 8);
-                        float f[8];
-                        unpack8<DT>(vv, f);
-                        const V p = reinterpret_cast<const V*>(pres)[rr];
-#pragma unroll
-                        for (int k = 0; k < 8; ++k)
-#pragma unroll
-                            for (int h = 0; h < HPB; ++h) accv[k][h] += p.v[h] * f[k];
-                    }
-                }
+                if (more) load_res_v(r0 + kResTile, rv);   // next tile's V slices, in place
             }
             // fold the row slots: 4 per wave (lane bits 4,5), then the waves
 #pragma unroll
             for (int k = 0; k < 8; ++k)
 #pragma unroll
-                for (int h = 0; h < HPB; ++h) {
-                    accv[k][h] += __shfl_xor(accv[k][h], 16, kWave);
-                    accv[k][h] += __shfl_xor(accv[k][h], 32, kWave);
-                }
+                for (int h = 0; h < HPB; ++h) accv[k][h] = quad_reduce(accv[k][h], OpSum(), 0.f);
             __syncthreads();
             float* red2 = reinterpret_cast<float*>(regA);  // [wave][kD][HPB]
-            if (lane < 16) {
+            if ((lane & 3) == 0) {
 #pragma unroll
                 for (int k = 0; k < 8; ++k)
 #pragma unroll
@@ -571,15 +765,12 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
             }
         }
 
-        // ---- phase 6: merge / write -------------------------------------------------
+        // ---- phase 6: merge / write ---------------------------------------------------------
+        __syncthreads();
         if (tid < HPB * kD) {
             const int h = tid / kD, d = tid % kD;
-            float mi = m_img[0], li = l_img[0], mr = m_res[0], lr = l_res[0];
-#pragma unroll
-            for (int k = 1; k < HPB; ++k) {
-                mi = (h == k) ? m_img[k] : mi; li = (h == k) ? l_img[k] : li;
-                mr = (h == k) ? m_res[k] : mr; lr = (h == k) ? l_res[k] : lr;
-            }
+            const float mr = stat[HPB + h], lr = stat[2 * HPB + h];
+            const float mi = stat[3 * HPB + h], li = stat[4 * HPB + h];
             const int64_t row = static_cast<int64_t>(b) * g.Hq + hq0 + h;
             if (g.nsplit == 1) {
                 const float mf = fmaxf(mi, mr);
@@ -595,7 +786,6 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                 p[2 + d] = is_img ? o_img : o_res;
             }
         }
-        (void)bc;
     }
 }
 
@@ -698,6 +888,7 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
     if (g.nsplit > 1) {
         DecodeGeom g1 = g;
         g1.nx = g.nsplit;  // the min/max pass has no residual unit
+        g1.cap = 0;        // ... and keeps no logits
         const int lds_mm = Lay<BITS, HPB>::lds_bytes(0);
         hipLaunchKernelGGL(kmm, dim3(units * g.nsplit), dim3(kNT), lds_mm, st, g1);
         CQ_LAUNCH_CHECK();
@@ -761,6 +952,7 @@ int cq_decode_attn(const cq_decode_args* a, cq_stream_t stream) {
     g.nsplit = p.nsplit; g.chunk = p.chunk; g.nx = p.nx;
     g.calib = a->calibrate; g.off_max = a->calib_off_max; g.off_min = a->calib_off_min;
     g.cap = p.cap;
+    g.one = 1.0f;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (a->dtype == CQ_BF16) return cq::dispatch<cq::BF16>(g, p, a->bits, st);
     return cq::dispatch<cq::FP16>(g, p, a->bits, st);
