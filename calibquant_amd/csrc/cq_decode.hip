@@ -15,9 +15,9 @@
 //            in place in LDS.
 //   V side   tokens are taken four at a time: a 16-entry table of subset sums
 //            of their e values is built once per group, every byte column of
-//            the packed V rows is bit-transposed with 256-entry spread tables
-//            (one per token position, pre-shifted to table offsets), and each
-//            of the 8 bit lanes of the column adds one table entry.  Scale /
+//            the packed V rows is staged byte-transposed (the 4 tokens' bytes of a
+//            column in one dword), a 4-byte dot product turns each bit lane of the
+//            column into a table offset, and the lane adds that table entry.  Scale /
 //            zero-point are applied once at the end.
 //   residual the full-precision rows run as an online-softmax flash-decode in
 //            the same workgroup (packed dot2 for q.K) and are merged at the end.
@@ -40,6 +40,7 @@ constexpr int kNW = kNT / kWave;   // waves per workgroup
 constexpr int kPF = 4;             // 16-byte loads kept in flight per thread and stream
 constexpr int kResTile = kNT / 8;  // residual rows per tile (8 lanes per row)
 constexpr int kLdsMax = 160 * 1024;
+constexpr float kLog2e = 1.4426950408889634f;
 
 template <int N> struct alignas(N * 4) Vec { float v[N]; };
 // native 16-byte vector: copies are single vector moves (HIP's uint4 struct copies lower to memcpy)
@@ -72,12 +73,12 @@ template <int BITS, int HPB> struct Lay {
     static constexpr int NB = 16 * BITS;            // bytes per packed row
     static constexpr int PC = NB * 8;               // bit lanes per row
     static constexpr int GPW = kWave / NB;          // 4-token groups per wave pass
+    static constexpr int MPL = 8 / GPW;             // bit lanes of a byte column handled by one lane
     static constexpr int TPW = 4 * GPW;             // tokens per wave pass
     static constexpr int ESZ = HPB * 4;             // bytes per fp32 table entry / logits slot
     static constexpr int HW = HPB >= 2 ? HPB / 2 : 1;   // 32-bit words per packed-fp16 entry
     static constexpr int ESZH = HW * 4;             // bytes per packed-fp16 table entry
     static constexpr int KT = NB * 256 * ESZ;       // K table bytes
-    static constexpr int SPREAD = 4 * 256 * 8;      // four spread tables
     static constexpr int WTAB = kNW * GPW * 16 * ESZH;
     static constexpr int VSUB = kNT * kPF / BITS;   // V tokens staged at a time
     static constexpr int KR = kPF / BITS;           // K token rounds in flight per thread
@@ -97,7 +98,7 @@ template <int BITS, int HPB> struct Lay {
     static constexpr int F_END = F_PRES + kResTile * HPB;
     static constexpr int FIXED = ((F_END * 4 + 255) / 256) * 256;
     static constexpr int region_a(int cap) {
-        return (cmax(cmax(KT, SPREAD + WTAB + cmin(VSUB, cap) * NB), cmax(RED, RED2)) + 255) / 256 * 256;
+        return (cmax(cmax(KT, WTAB + cmin(VSUB, cap) * NB), cmax(RED, RED2)) + 255) / 256 * 256;
     }
     static constexpr int lds_bytes(int cap) { return region_a(cap) + FIXED + cap * ESZ; }
     static constexpr int max_chunk() {
@@ -151,19 +152,6 @@ template <> __device__ __forceinline__ float dot2<FP16>(uint32_t a, uint32_t b, 
 }
 
 template <int N> struct alignas(N * 4) Words { uint32_t w[N]; };
-
-// x + (x of lane ^ 16) and x + (x of lane ^ 32) with the row / half-wave swap
-// instructions: a copy is swapped against the original, then the pair is added.
-__device__ __forceinline__ float add_lane_xor16(float x) {
-    uint32_t a = __builtin_bit_cast(uint32_t, x), b;
-    asm volatile("v_mov_b32 %1, %0\n\ts_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "=&v"(b));
-    return __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b);
-}
-__device__ __forceinline__ float add_lane_xor32(float x) {
-    uint32_t a = __builtin_bit_cast(uint32_t, x), b;
-    asm volatile("v_mov_b32 %1, %0\n\ts_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "=&v"(b));
-    return __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b);
-}
 
 __device__ __forceinline__ uint32_t pack_f16(float a, float b) {
     f16x2_t h = {static_cast<_Float16>(a), static_cast<_Float16>(b)};   // round to nearest even
@@ -410,9 +398,9 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
         if constexpr (L::KR > (R)) {                                                          \
             token_logits(tid + (R) * kNT, kc[(R)]);                                           \
             if constexpr (!MINMAX_ONLY) {                                                     \
-                vc[(R) * BITS] = cvp4[min(tid + ((R) * BITS) * kNT, last_u)];                 \
+                vc[(R) * BITS] = cvp4[min((tid + (R) * kNT) * BITS, last_u)];                 \
                 if constexpr (BITS == 2)                                                      \
-                    vc[(R) * BITS + 1] = cvp4[min(tid + ((R) * BITS + 1) * kNT, last_u)];     \
+                    vc[(R) * BITS + 1] = cvp4[min((tid + (R) * kNT) * BITS + 1, last_u)];     \
             }                                                                                 \
         }
         CQ_K_ROUND(0)
@@ -454,28 +442,37 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
         float o_img = 0.f;  // thread (h, d) = (tid / kD, tid % kD) for tid < HPB*kD
 
         if (n > 0) {
-            // the K table is dead: stage the first block of packed V rows and the
-            // spread tables in its place (ordered by the barriers of block_reduce)
-            uint2* spread = reinterpret_cast<uint2*>(regA);
-            unsigned char* vst = regA + L::SPREAD + L::WTAB;
-            {
-                const int c = tid & 255, pos = tid >> 8;   // kNT == 4 * 256
-                uint32_t lo = 0, hi = 0;
+            // The K table is dead: stage the first block of packed V rows in its place
+            // (ordered by the barriers of block_reduce).  Layout: [unit of TPW tokens]
+            // [byte column][token], so the 4 bytes that the 4 tokens of a group have in one
+            // column form one dword.  A quad of lanes holds a group (tokens are
+            // lane-consecutive): each lane gathers, for 4 of the 16 columns of its 16-byte
+            // piece, the 4 tokens' bytes with quad broadcasts and byte permutes.
+            unsigned char* vst = regA + L::WTAB;
+            const int qi = lane & 3;
+            const uint32_t sel_pair = static_cast<uint32_t>(qi) | (static_cast<uint32_t>(4 + qi) << 8) | 0x0c0c0000u;
+            auto stage_piece = [&](U4 c, int tok, int piece, bool write) {
+                const uint32_t w[4] = {c.x, c.y, c.z, c.w};
+                const int base = ((tok / L::TPW) * NB + 16 * piece + qi) * L::TPW + ((tok % L::TPW) & ~3);
 #pragma unroll
-                for (int m = 0; m < 4; ++m) {
-                    lo |= ((c >> (7 - m)) & 1u) << (8 * m);
-                    hi |= ((c >> (3 - m)) & 1u) << (8 * m);
+                for (int q = 0; q < 4; ++q) {
+                    const int wi = static_cast<int>(w[q]);
+                    const uint32_t x0 = __builtin_amdgcn_update_dpp(0, wi, 0x00, 0xf, 0xf, false);
+                    const uint32_t x1 = __builtin_amdgcn_update_dpp(0, wi, 0x55, 0xf, 0xf, false);
+                    const uint32_t x2 = __builtin_amdgcn_update_dpp(0, wi, 0xAA, 0xf, 0xf, false);
+                    const uint32_t x3 = __builtin_amdgcn_update_dpp(0, wi, 0xFF, 0xf, 0xf, false);
+                    const uint32_t lo = __builtin_amdgcn_perm(x1, x0, sel_pair);
+                    const uint32_t hi = __builtin_amdgcn_perm(x3, x2, sel_pair);
+                    const uint32_t t4 = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+                    if (write) *reinterpret_cast<uint32_t*>(vst + base + 4 * q * L::TPW) = t4;
                 }
-                constexpr int esh = L::ESZH == 8 ? 3 : 2;
-                spread[pos * 256 + c] = make_uint2(lo << (esh + pos), hi << (esh + pos));
-            }
-
+            };
             {
                 const int vn0 = min(L::VSUB, npad);
 #pragma unroll
                 for (int r = 0; r < kPF; ++r) {
-                    const int u = tid + r * kNT;
-                    if (u < vn0 * NB / 16) reinterpret_cast<U4*>(vst)[u] = vc[r];
+                    const int tok = tid + (r / BITS) * kNT;
+                    stage_piece(vc[r], tok, r % BITS, tok < vn0);
                 }
             }
 
@@ -534,7 +531,7 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
 #pragma unroll
                     for (int h = 0; h < HPB; ++h) {
                         const float x = (w.v[h] - mn[h]) * slope[h] + tmin[h];
-                        e[h] = (m_img[h] == -INFINITY) ? 0.f : __expf(x - m_img[h]);
+                        e[h] = (m_img[h] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((x - m_img[h]) * kLog2e);
                         ls[h] += e[h];
                     }
                 }
@@ -544,13 +541,14 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                 if constexpr (L::HW == 2) hw.w[1] = pack_f16(e[2], e[3]);
                 *reinterpret_cast<HWv*>(&logits[tt]) = hw;
             }
-            block_reduce<HPB>(ls, red, OpSum(), 0.f);   // its barriers also publish e, spread, vst
+            block_reduce<HPB>(ls, red, OpSum(), 0.f);   // its barriers also publish e and vst
 #pragma unroll
             for (int h = 0; h < HPB; ++h) l_img[h] = ls[h];
 
             // ---- phase 4: packed V ----------------------------------------------------------
-            unsigned char* wtab = regA + L::SPREAD + wv * (L::GPW * 16 * L::ESZH);
-            const int j = lane % NB, gs = lane / NB;
+            // lane = (byte column j, slice c of its 8 bit lanes); a wave pass covers TPW tokens
+            unsigned char* wtab = regA + wv * (L::GPW * 16 * L::ESZH);
+            const int j = lane / L::GPW, cs = lane % L::GPW;
             const int bg = lane >> 4, be = lane & 15;   // table build: group, entry
             f16x2_t bsel[4];
 #pragma unroll
@@ -558,22 +556,29 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                 const _Float16 f = static_cast<_Float16>(static_cast<float>((be >> i) & 1));
                 bsel[i] = f16x2_t{f, f};
             }
-            float acc[8][HPB];
+            float acc[L::MPL][HPB];
 #pragma unroll
-            for (int m = 0; m < 8; ++m)
+            for (int m = 0; m < L::MPL; ++m)
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) acc[m][h] = 0.f;
             const float one = g.one;
+            // bit lane m of the byte is bit 7 - m; entry offset = sum_i bit(token i) * ESZH * 2^i
+            uint32_t shr[L::MPL];
+#pragma unroll
+            for (int m = 0; m < L::MPL; ++m) shr[m] = 7 - (cs * L::MPL + m);
+            constexpr uint32_t kMult = L::ESZH * 0x08040201u;
+            using WG = Words<L::GPW>;   // the GPW dwords of one (unit, column)
+            const uint32_t wtab_addr = static_cast<uint32_t>(wtab - smem);   // byte offset in LDS
 
             for (int vs0 = 0; vs0 < npad; vs0 += L::VSUB) {
                 const int vn = min(L::VSUB, npad - vs0);
                 if (vs0 > 0) {
                     __syncthreads();  // previous block consumed
-                    for (int u = tid; u < vn * NB / 16; u += kNT) {
-                        const int tok = vs0 + u * 16 / NB;
-                        uint4 c = make_uint4(0, 0, 0, 0);
-                        if (tok < n) c = cvp[static_cast<int64_t>(vs0) * NB / 16 + u];
-                        reinterpret_cast<uint4*>(vst)[u] = c;
+#pragma unroll
+                    for (int r = 0; r < kPF; ++r) {
+                        const int tok = tid + (r / BITS) * kNT;
+                        const U4 c = cvp4[min((vs0 + tok) * BITS + r % BITS, last_u)];
+                        stage_piece(c, tok, r % BITS, tok < vn);
                     }
                     __syncthreads();
                 }
@@ -595,51 +600,38 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                         for (int k = 0; k < L::HW; ++k) o.w[k] = __builtin_bit_cast(uint32_t, val[k]);
                         reinterpret_cast<HWv*>(wtab)[bg * 16 + be] = o;
                     }
-                    uint32_t xlo = 0, xhi = 0;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const uint32_t c = vst[(tl + 4 * gs + i) * NB + j];
-                        const uint2 sp = spread[i * 256 + c];
-                        xlo |= sp.x;
-                        xhi |= sp.y;
-                    }
+                    const WG cw = *reinterpret_cast<const WG*>(vst + (u * NB + j) * L::TPW);
                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                     __builtin_amdgcn_wave_barrier();
                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-                    const unsigned char* tbp = wtab + gs * (16 * L::ESZH);
 #pragma unroll
-                    for (int m = 0; m < 8; ++m) {
-                        const uint32_t x = m < 4 ? xlo : xhi;
-                        const HWv e = *reinterpret_cast<const HWv*>(tbp + ((x >> (8 * (m & 3))) & 0xffu));
+                    for (int gq = 0; gq < L::GPW; ++gq) {
+                        const uint32_t tbase = wtab_addr + static_cast<uint32_t>(gq * 16 * L::ESZH);
 #pragma unroll
-                        for (int h = 0; h < HPB; ++h) {
-                            const f16x2_t pr = __builtin_bit_cast(f16x2_t, e.w[h >> 1]);
-                            const _Float16 hv = (h & 1) ? pr.y : pr.x;
-                            acc[m][h] = __builtin_fmaf(static_cast<float>(hv), one, acc[m][h]);
+                        for (int m = 0; m < L::MPL; ++m) {
+                            const uint32_t bits = (cw.w[gq] >> shr[m]) & 0x01010101u;
+                            const uint32_t off = __builtin_amdgcn_udot4(bits, kMult, tbase, false);
+                            const HWv e = *reinterpret_cast<const HWv*>(smem + off);
+#pragma unroll
+                            for (int h = 0; h < HPB; ++h) {
+                                const f16x2_t pr = __builtin_bit_cast(f16x2_t, e.w[h >> 1]);
+                                const _Float16 hv = (h & 1) ? pr.y : pr.x;
+                                acc[m][h] = __builtin_fmaf(static_cast<float>(hv), one, acc[m][h]);
+                            }
                         }
                     }
                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                     __builtin_amdgcn_wave_barrier();
                 }
             }
-            // fold the group slots of the wave, then the waves
-#pragma unroll
-            for (int m = 0; m < 8; ++m)
-#pragma unroll
-                for (int h = 0; h < HPB; ++h) {
-                    if constexpr (L::GPW == 4) acc[m][h] = add_lane_xor16(acc[m][h]);
-                    acc[m][h] = add_lane_xor32(acc[m][h]);
-                }
             __syncthreads();
             V* redv = reinterpret_cast<V*>(regA);  // [wave][PC]
-            if (gs == 0) {
 #pragma unroll
-                for (int m = 0; m < 8; ++m) {
-                    V a4;
+            for (int m = 0; m < L::MPL; ++m) {
+                V a4;
 #pragma unroll
-                    for (int h = 0; h < HPB; ++h) a4.v[h] = acc[m][h];
-                    redv[wv * L::PC + j * 8 + m] = a4;
-                }
+                for (int h = 0; h < HPB; ++h) a4.v[h] = acc[m][h];
+                redv[wv * L::PC + j * 8 + cs * L::MPL + m] = a4;
             }
             __syncthreads();
             if (tid < HPB * kD) {
@@ -740,7 +732,7 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                     for (int k = 0; k < 8; ++k)
 #pragma unroll
                         for (int h = 0; h < HPB; ++h)
-                            accv[k][h] = (rep == 0 ? accv[k][h] * alpha[h] : accv[k][h]) + p.v[h] * f[k];
+                            accv[k][h] = ((rep == 0 && r0 > 0) ? accv[k][h] * alpha[h] : accv[k][h]) + p.v[h] * f[k];
                 }
                 if (more) load_res_v(r0 + kResTile, rv);   // next tile's V slices, in place
             }
