@@ -1,0 +1,244 @@
+"""The reference's `patch_internvl.py` surface for the CalibQuant method, routed to
+the MI355X kernels: `patch_model`, `ATTN_FORWARD_FUNCTIONS`, `custom_generate`,
+`forward_internlm2_calibquant`, the RoPE / GQA helpers and the module constants.
+
+What changes behind the same call contract (patch_internvl.py:141-150, 484):
+  * prefill: the image slice of K and V is quantised and packed by one HIP entry
+    point per tensor, reading the strided views of the fused wqkv output in place
+    (reference: quant + unique/compare/argmax + encode, patch_internvl.py:288-341);
+  * decode: one fused HIP call replaces repeat_kv copies, two Triton LUT vec-mats,
+    the calibration, softmax and residual matmuls (patch_internvl.py:344-436);
+  * the fp residual window is appended in place instead of `torch.cat` per step
+    (patch_internvl.py:264-266); callers still get and pass plain (K, V) tensors.
+The QJL method of the reference (`quant_method='qjl'`) is a different algorithm
+and is not provided.
+"""
+from __future__ import annotations
+
+import os
+import warnings
+from typing import Optional, Tuple
+
+import torch
+
+from . import ops
+from ._lib import CalibQuantError
+from .kvbuffer import GrowingKV
+
+# global hyper-parameters, as in patch_internvl.py:19-31
+BITS_KV = 1
+
+if BITS_KV == 1:
+    SCALE_V = 0.3
+    SCALE_K = 0.5
+else:
+    SCALE_V = 1
+    SCALE_K = 1
+
+LOW_BITS = True
+SPROMPT_LEN = 41
+CHUNK_SIZE = 1024
+CALIB_OFFSET_MAX = -3.0    # literals at patch_internvl.py:379-380
+CALIB_OFFSET_MIN = 0.0
+
+
+def repeat_kv(hidden_states: torch.Tensor, n_rep: int) -> torch.Tensor:
+    """(B, Hkv, S, D) -> (B, Hkv * n_rep, S, D), each kv head repeated consecutively (patch_internvl.py:97-107)."""
+    b, h, s, d = hidden_states.shape
+    if n_rep == 1:
+        return hidden_states
+    return hidden_states[:, :, None, :, :].expand(b, h, n_rep, s, d).reshape(b, h * n_rep, s, d)
+
+
+def rotate_half(x):
+    """(-x2, x1) for x = (x1, x2) split along the last axis (patch_internvl.py:110-115; this version
+    leaves its argument untouched)."""
+    h = x.shape[-1] // 2
+    return torch.cat((-x[..., h:], x[..., :h]), dim=-1)
+
+
+def apply_rotary_pos_emb(q, k, cos, sin, position_ids, unsqueeze_dim=1):
+    """Rotary position embedding of q and k (patch_internvl.py:119-138)."""
+    cos = cos[position_ids].unsqueeze(unsqueeze_dim)
+    sin = sin[position_ids].unsqueeze(unsqueeze_dim)
+    return (q * cos) + (rotate_half(q) * sin), (k * cos) + (rotate_half(k) * sin)
+
+
+@torch.no_grad()
+def custom_generate(self, pixel_values=None, input_ids=None, attention_mask=None, visual_features=None,
+                    generation_config=None, output_hidden_states=None, **generate_kwargs):
+    """`InternVLChatModel.generate` replacement (patch_internvl.py:34-93): vision features in chunks
+    of 10 tiles, splice them over the image-context tokens, publish the per-sample image token count,
+    run the language model's generate."""
+    assert self.img_context_token_id is not None
+    lm = self.language_model
+    if pixel_values is not None:
+        if visual_features is not None:
+            vit_embeds = visual_features
+        else:
+            chunks = [self.extract_feature(pixel_values[i:i + 10]) for i in range(0, pixel_values.size(0), 10)]
+            vit_embeds = torch.cat(chunks, dim=0)
+        input_embeds = lm.get_input_embeddings()(input_ids)
+        B, N, C = input_embeds.shape
+        input_embeds = input_embeds.reshape(B * N, C)
+        selected = input_ids.reshape(B * N) == self.img_context_token_id
+        assert selected.sum() != 0
+        input_embeds[selected] = vit_embeds.reshape(-1, C).to(input_embeds.device, input_embeds.dtype)
+        image_token_num = int(vit_embeds.shape[0] * vit_embeds.shape[1] / B)
+        os.environ["IMAGE_TOKEN_NUM"] = str(image_token_num)
+        for layer in lm.model.layers:
+            layer.attention.image_token_num = image_token_num
+        input_embeds = input_embeds.reshape(B, N, C)
+    else:
+        input_embeds = lm.get_input_embeddings()(input_ids)
+    return lm.generate(inputs_embeds=input_embeds, attention_mask=attention_mask,
+                       generation_config=generation_config, output_hidden_states=output_hidden_states,
+                       use_cache=True, **generate_kwargs)
+
+
+def _image_token_num(self) -> int:
+    n = getattr(self, "image_token_num", None)
+    if n is None:
+        env = os.environ.get("IMAGE_TOKEN_NUM")
+        if env is None:
+            raise CalibQuantError("image token count unknown: set attention.image_token_num or IMAGE_TOKEN_NUM")
+        n = int(env)
+    return int(n)
+
+
+def forward_internlm2_calibquant(self, hidden_states: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
+                                 position_ids: Optional[torch.LongTensor] = None,
+                                 past_key_value: Optional[Tuple[torch.Tensor]] = None,
+                                 output_attentions: bool = False, use_cache: bool = False, **kwargs):
+    """Attention forward with a 1-/2-bit image KV cache (patch_internvl.py:141-484).
+
+    Returns `(attn_output, None, past_key_value)`; `past_key_value` is the fp pair
+    (K, V) of shape (B, Hkv, R, D) holding the system prompt rows [0, S), the text rows and every
+    generated token; the image rows live packed on the module
+    (`encoded_features_k/v`, `scale_key/value`, `zero_point_key/value`, `unique_values_k/v`)."""
+    # hyper-parameters published on the module, as patch_internvl.py:175-191 does
+    self.sprompt_len = getattr(self, "cq_sprompt_len", SPROMPT_LEN)
+    self.bits_k = self.bits_v = getattr(self, "cq_bits", BITS_KV)
+    one_bit = self.bits_k == 1
+    self.scale_k = getattr(self, "cq_scale_k", 0.5 if one_bit else 1)
+    self.scale_v = getattr(self, "cq_scale_v", 0.3 if one_bit else 1)
+    self.per_channel_k = self.per_channel_v = True
+    self.image_token_num = _image_token_num(self)
+    self.normalize = self.bits_k <= 2
+    if "padding_mask" in kwargs:
+        warnings.warn("Passing `padding_mask` is deprecated; use `attention_mask` instead.")
+        attention_mask = kwargs.pop("padding_mask")
+
+    bsz, q_len, _ = hidden_states.size()
+    G, D, Hq = self.num_key_value_groups, self.head_dim, self.num_heads
+    Hkv = Hq // G
+    S, T = self.sprompt_len, self.image_token_num
+
+    # (h gs d) de-interleave of the fused projection: views only (patch_internvl.py:214-234)
+    qkv = self.wqkv(hidden_states).view(bsz, q_len, Hkv, 2 + G, D)
+    query_states = qkv[..., :G, :].reshape(bsz, q_len, Hq, D).transpose(1, 2)     # (B, Hq, q, D)
+    key_states = qkv[..., -2, :].transpose(1, 2)                                   # (B, Hkv, q, D)
+    value_states = qkv[..., -1, :].transpose(1, 2)
+
+    kv_seq_len = q_len
+    if past_key_value is not None:
+        kv_seq_len += past_key_value[0].shape[-2] + T                               # patch_internvl.py:246-251
+    cos, sin = self.rotary_emb(value_states, seq_len=kv_seq_len)
+    query_states, key_states = apply_rotary_pos_emb(query_states, key_states, cos, sin, position_ids)
+
+    if not hasattr(self, "_cq_window"):
+        self._cq_window = GrowingKV()
+
+    if q_len > 1:
+        # ---- prefill (patch_internvl.py:268-341, 461-476) -------------------------------------
+        if past_key_value is not None:
+            raise CalibQuantError("prefill with an existing cache is not supported (the reference quantises "
+                                  "the image block of a fresh prompt)")
+        if S + T > q_len:
+            raise CalibQuantError(f"prompt of {q_len} tokens is shorter than sprompt_len + image tokens = {S + T}")
+        if T > 0:
+            k_img = key_states[:, :, S:S + T, :].transpose(1, 2)      # (B, T, Hkv, D) strided views
+            v_img = value_states[:, :, S:S + T, :].transpose(1, 2)
+            ck, ks, kz = ops.quantize_pack(k_img, self.bits_k, self.scale_k)
+            cv, vs, vz = ops.quantize_pack(v_img, self.bits_v, self.scale_v)
+            self.encoded_features_k, self.encoded_features_v = ck, cv
+            self._cq_stats = (ks, kz, vs, vz)                          # compact (B, Hkv, D)
+            # reference-shaped views of the statistics: (B, Hq, 1, D) after repeat_kv (patch_internvl.py:300-309)
+            self.scale_key = repeat_kv(ks.unsqueeze(2), G)
+            self.zero_point_key = repeat_kv(kz.unsqueeze(2), G)
+            self.scale_value = repeat_kv(vs.unsqueeze(2), G)
+            self.zero_point_value = repeat_kv(vz.unsqueeze(2), G)
+            lut = torch.arange(2 ** self.bits_k, device=hidden_states.device, dtype=hidden_states.dtype)
+            self.unique_values_k, self.unique_values_v = lut, lut.half()
+        else:
+            self.encoded_features_k = self.encoded_features_v = None
+            self._cq_stats = None
+        if use_cache:
+            k_st = torch.cat([key_states[:, :, :S], key_states[:, :, S + T:]], dim=2)
+            v_st = torch.cat([value_states[:, :, :S], value_states[:, :, S + T:]], dim=2)
+            self._cq_window = GrowingKV()
+            past_key_value = self._cq_window.append(None, k_st, v_st)
+        else:
+            past_key_value = None
+        # full-precision causal attention over the whole prompt, in query chunks
+        q_t, k_t, v_t = query_states.transpose(1, 2), key_states.transpose(1, 2), value_states.transpose(1, 2)
+        outs = []
+        for i in range(0, q_len, CHUNK_SIZE):
+            outs.append(self._flash_attention_forward(q_t[:, i:i + CHUNK_SIZE], k_t[:, :i + CHUNK_SIZE],
+                                                      v_t[:, :i + CHUNK_SIZE], attention_mask if attention_mask is None
+                                                      or attention_mask.dim() == 2 else None,
+                                                      q_t[:, :i + CHUNK_SIZE].shape[1]))
+        attn_output = torch.cat(outs, dim=1).reshape(bsz, q_len, self.hidden_size)
+        return self.wo(attn_output), None, past_key_value
+
+    # ---- decode (patch_internvl.py:344-457) -------------------------------------------------------
+    k_res, v_res = self._cq_window.append(past_key_value, key_states, value_states)
+    past_key_value = (k_res, v_res) if use_cache else None
+    R = k_res.shape[2]
+    if kv_seq_len != R + T:
+        raise ValueError(f"Attention weights should be of size {(bsz, Hq, q_len, kv_seq_len)}, but is "
+                         f"{(bsz, Hq, q_len, R + T)}")
+    mask = None
+    if attention_mask is not None:
+        if attention_mask.size() != (bsz, 1, q_len, kv_seq_len):
+            raise ValueError(f"Attention mask should be of size {(bsz, 1, q_len, kv_seq_len)}, "
+                             f"but is {attention_mask.size()}")
+        mask = attention_mask[:, 0, 0, :]
+    stats = self._cq_stats if T > 0 else (None,) * 4
+    out = ops.decode_attn(query_states[:, :, 0, :], self.encoded_features_k if T > 0 else None,
+                          self.encoded_features_v if T > 0 else None, stats[0], stats[1], stats[2], stats[3],
+                          k_res, v_res, sprompt_len=min(S, R), bits=self.bits_k, calibrate=self.normalize,
+                          calib_off_max=CALIB_OFFSET_MAX, calib_off_min=CALIB_OFFSET_MIN, mask=mask)
+    attn_output = self.wo(out.reshape(bsz, 1, self.hidden_size))
+    return attn_output, None, past_key_value
+
+
+def _no_qjl(*args, **kwargs):
+    raise CalibQuantError("quant_method='qjl' (the QJL sketch method) is not part of this build; use 'calibquant'")
+
+
+ATTN_FORWARD_FUNCTIONS = {
+    "calibquant": forward_internlm2_calibquant,
+    "qjl": _no_qjl,
+}
+
+
+def patch_model(model, quant_method="calibquant", **kwargs):
+    """Route a chat model's generate and its attention forward to the quantised-KV path
+    (patch_internvl.py:645-660).  Works on any object exposing
+    `language_model.model.layers[i].attention` and a class-level `generate`.
+    Optional keyword overrides: bits, scale_k, scale_v, sprompt_len."""
+    if quant_method not in ATTN_FORWARD_FUNCTIONS:
+        raise KeyError(quant_method)
+    if quant_method == "qjl":
+        _no_qjl()
+    print("Patching InternVLChatModel.generate function ...")
+    model.__class__.generate = custom_generate
+    print(f"Patching InternLM2FlashAttention2.forward function ... {quant_method}")
+    layers = model.language_model.model.layers
+    layers[0].attention.__class__.forward = ATTN_FORWARD_FUNCTIONS[quant_method]
+    for name in ("bits", "scale_k", "scale_v", "sprompt_len"):
+        if name in kwargs:
+            for layer in layers:
+                setattr(layer.attention, "cq_" + name, kwargs[name])
+    return model

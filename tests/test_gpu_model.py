@@ -1,0 +1,123 @@
+"""The patched attention forward / model routing on the GPU: cache bookkeeping,
+prefill quantisation of the strided wqkv views, decode through the fused kernel."""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cq_oracle as O
+from tests.util import to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def _tiny_model(layers=2, seed=0):
+    from calibquant_amd.internlm2 import InternLM2Config, InternVLChatStandIn
+    torch.manual_seed(seed)
+    m = InternVLChatStandIn(InternLM2Config.tiny(layers)).cuda().to(torch.bfloat16).eval()
+    return m
+
+
+def test_patched_forward_decode_matches_oracle_on_one_layer():
+    """Prefill S + T + text tokens, then one decode step: the layer's attention output equals
+    wo(oracle attention) built from the module's own packed state and fp window."""
+    from calibquant_amd import patch_internvl as pi
+    from calibquant_amd.internlm2 import InternLM2Attention, InternLM2Config
+    torch.manual_seed(1)
+    cfg = InternLM2Config.tiny()
+    att = InternLM2Attention(cfg).cuda().to(torch.bfloat16)
+    att.cq_sprompt_len, att.image_token_num = 5, 200
+    B, S, T, TXT = 2, 5, 200, 11
+    N = S + T + TXT
+    x = torch.randn(B, N, cfg.hidden_size, device="cuda", dtype=torch.bfloat16)
+    pos = torch.arange(N, device="cuda")[None].expand(B, N)
+    with torch.no_grad():
+        out_p, _, past = pi.forward_internlm2_calibquant(att, x, None, pos, None, False, True)
+        assert out_p.shape == (B, N, cfg.hidden_size)
+        assert past[0].shape == (B, cfg.num_key_value_heads, S + TXT, 128)
+        assert att.encoded_features_k.shape == (B, cfg.num_key_value_heads, T, 16)
+        assert att.scale_key.shape == (B, cfg.num_attention_heads, 1, 128)
+        # the packed state equals the oracle's quantisation of the post-RoPE image keys / raw values
+        q, k, v = att.split_qkv(x)
+        cos, sin = att.rotary_emb(v, seq_len=N)
+        qr, kr = pi.apply_rotary_pos_emb(q.transpose(1, 2), k.transpose(1, 2), cos, sin, pos)
+        ck, sk, zk = O.quantize_pack(to_np(kr[:, :, S:S + T].transpose(1, 2)), 1, 0.5, "bf16")
+        cv, sv, zv = O.quantize_pack(to_np(v[:, S:S + T]), 1, 0.3, "bf16")
+        assert np.array_equal(att.encoded_features_k.cpu().numpy(), ck)
+        assert np.array_equal(att.encoded_features_v.cpu().numpy(), cv)
+        # one decode step with an additive mask that hides two positions
+        xd = torch.randn(B, 1, cfg.hidden_size, device="cuda", dtype=torch.bfloat16)
+        posd = torch.full((B, 1), N, device="cuda", dtype=torch.long)
+        mask = torch.zeros(B, 1, 1, N + 1, device="cuda", dtype=torch.bfloat16)
+        mask[0, 0, 0, 2] = mask[1, 0, 0, S + 7] = torch.finfo(torch.bfloat16).min
+        out_d, _, past2 = pi.forward_internlm2_calibquant(att, xd, mask, posd, past, False, True)
+        assert past2[0].shape[2] == S + TXT + 1 and past2[0].data_ptr() == past[0].data_ptr()
+        qd, kd, vd = att.split_qkv(xd)
+        cos, sin = att.rotary_emb(vd, seq_len=N + 1)
+        qd, kd = pi.apply_rotary_pos_emb(qd.transpose(1, 2), kd.transpose(1, 2), cos, sin, posd)
+        want = O.decode_attention(to_np(qd[:, :, 0]), ck, cv, sk, zk, sv, zv, to_np(past2[0]), to_np(past2[1]),
+                                  S, 1, mask=to_np(mask[:, 0, 0]))
+        want = torch.from_numpy(want).cuda().to(torch.bfloat16).reshape(B, 1, -1)
+        ref = att.wo(want)
+        err = (out_d.float() - ref.float()).abs()
+        assert err.max().item() < 2e-2 and err.mean().item() < 2e-3
+
+
+def test_patched_model_without_image_tokens_equals_the_fp_model():
+    """With zero packed tokens the quantised path is plain attention over the fp window."""
+    from calibquant_amd import patch_internvl as pi
+    from calibquant_amd.internlm2 import InternLM2Attention
+    from calibquant_amd.internlm2 import InternVLChatStandIn
+    m = _tiny_model()
+    lm = m.language_model
+    fp_forward, fp_generate = InternLM2Attention.forward, InternVLChatStandIn.generate
+    ids = torch.randint(0, 500, (2, 40), device="cuda")
+    nxt = torch.randint(0, 500, (2, 1), device="cuda")
+    pos = torch.arange(40, device="cuda")[None].expand(2, 40)
+    pos1 = torch.full((2, 1), 40, device="cuda", dtype=torch.long)
+
+    def two_steps():
+        emb = lm.get_input_embeddings()
+        l0, past = lm.forward_step(emb(ids), pos, None)
+        l1, past = lm.forward_step(emb(nxt), pos1, past)
+        return l0.float(), l1.float()
+
+    try:
+        with torch.no_grad():
+            b0, b1 = two_steps()
+            pi.patch_model(m, "calibquant", sprompt_len=0)
+            for layer in lm.model.layers:
+                layer.attention.image_token_num = 0
+            p0, p1 = two_steps()
+        assert torch.allclose(b0, p0, atol=3e-2, rtol=3e-2)
+        assert torch.allclose(b1, p1, atol=3e-2, rtol=3e-2)
+    finally:
+        InternLM2Attention.forward, InternVLChatStandIn.generate = fp_forward, fp_generate
+
+
+def test_patch_model_and_custom_generate_end_to_end():
+    """Two synthetic tiles per sample -> 512 image tokens, quantised at prefill, 8 greedy tokens."""
+    from calibquant_amd import patch_internvl as pi
+    from calibquant_amd.internlm2 import InternLM2Attention, InternVLChatStandIn
+    fp_forward, fp_generate = InternLM2Attention.forward, InternVLChatStandIn.generate
+    m = _tiny_model(seed=3)
+    B, S, tiles, txt = 2, 41, 2, 9
+    T = tiles * 256
+    ids = torch.randint(0, 500, (B, S + T + txt), device="cuda")
+    ids[:, S:S + T] = m.img_context_token_id
+    pix = torch.rand(B * tiles, 3, 448, 448, device="cuda", dtype=torch.bfloat16)
+    try:
+        pi.patch_model(m, "calibquant")
+        os.environ.pop("IMAGE_TOKEN_NUM", None)
+        out = m.generate(pixel_values=pix, input_ids=ids, max_new_tokens=8)
+        assert out.shape == (B, 8)
+        assert os.environ["IMAGE_TOKEN_NUM"] == str(T)
+        att = m.language_model.model.layers[0].attention
+        assert att.encoded_features_k.shape == (B, 2, T, 16) and att.encoded_features_k.dtype == torch.uint8
+        assert att._cq_window.len == S + txt + 7
+        out2 = m.generate(pixel_values=pix, input_ids=ids, max_new_tokens=8)
+        assert torch.equal(out, out2)
+    finally:
+        InternLM2Attention.forward, InternVLChatStandIn.generate = fp_forward, fp_generate

@@ -1,0 +1,90 @@
+"""GPU parity of the four operators of the reference's `calibquant.py` surface
+(quant, encode, fused_kernel, fused_kernel_wv) against the oracle, and of the
+unfused call sequence of the reference's decode branch assembled from them."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cq_oracle as O
+from tests.util import CLIPS, make_case, case_to_gpu, same_bits, to_gpu, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def cq():
+    from calibquant_amd import calibquant
+    return calibquant
+
+
+@pytest.mark.parametrize("bits", [1, 2])
+def test_quant_then_encode_like_the_reference_prefill(cq, bits):
+    """quant -> transpose -> (identity LUT) indices -> encode, patch_internvl.py:290-339."""
+    k, _ = O.synth_kv(2, 300, 4, 128, "bf16", seed=1)
+    x = to_gpu(k, "bf16")
+    x_q, s, z = cq.quant(x, bits=bits, per_channel=True, scale=CLIPS[bits][0], post_scale=True)
+    assert x_q.shape == x.shape and s.shape == (2, 1, 4, 128)
+    oxq, os_, oz = O.quant(k, bits, CLIPS[bits][0], "bf16")
+    assert same_bits(to_np(x_q), oxq) and same_bits(to_np(s), os_) and same_bits(to_np(z), oz)
+    idx = x_q.transpose(1, 2).long()                      # the reference's inverse_indices are int64
+    enc = cq.encode(idx, bits, 8 // bits)
+    assert enc.dtype == torch.uint8 and enc.shape == (2, 4, 300, 128 * bits // 8)
+    assert np.array_equal(enc.cpu().numpy(), O.encode(np.transpose(oxq, (0, 2, 1, 3)).astype(np.int64), bits))
+    deq, _, _ = cq.quant(x, bits=bits, per_channel=True, scale=CLIPS[bits][0], post_scale=False)
+    assert same_bits(to_np(deq), O.dequant(oxq, os_, oz, "bf16"))
+
+
+@pytest.mark.parametrize("bits", [1, 2])
+def test_fused_kernels_honour_an_arbitrary_table(cq, bits):
+    rng = np.random.default_rng(0)
+    B, H, T, D = 2, 8, 333, 128
+    idx = rng.integers(0, 2 ** bits, size=(B, H, T, D))
+    enc = O.encode(idx, bits)
+    lut = np.array([0.25, -1.5, 2.0, 3.0][: 2 ** bits], np.float32)
+    a = O.round_to(rng.standard_normal((B, H, 1, D)), "bf16")
+    p = O.round_to(rng.random((B, H, 1, T)) / T, "fp16")
+    enc_g = torch.from_numpy(enc).cuda()
+    qk = cq.fused_kernel(to_gpu(lut, "bf16"), to_gpu(a, "bf16"), enc_g, bits, 8 // bits)
+    pv = cq.fused_kernel_wv(to_gpu(lut, "fp16"), to_gpu(p, "fp16"), enc_g, bits, 8 // bits)
+    assert qk.dtype == torch.float16 and qk.shape == (B, H, 1, T) and pv.shape == (B, H, 1, D)
+    want_qk, want_pv = O.lut_vecmat_qk(lut, a, enc, bits), O.lut_vecmat_pv(lut, p, enc, bits)
+    # fp32 accumulation order differs from numpy's: allow one fp16 ulp
+    assert np.allclose(to_np(qk), want_qk, rtol=2e-3, atol=2e-3)
+    assert np.allclose(to_np(pv), want_pv, rtol=2e-3, atol=1e-4)
+
+
+def test_unfused_reference_sequence_agrees_with_the_fused_kernel(cq):
+    """The decode branch written as the reference writes it (patch_internvl.py:352-436), on top of
+    the four operators, lands within the reference's own mixed-precision noise of the fused kernel."""
+    from calibquant_amd import ops
+    from calibquant_amd.patch_internvl import repeat_kv
+    B, Hq, Hkv, T, R, S, bits = 2, 32, 8, 1024, 64, 41, 1
+    c = make_case(B, Hq, Hkv, 128, T, R, bits, "bf16", seed=3)
+    g = case_to_gpu(c, "bf16")
+    G = Hq // Hkv
+    q = g["q"][:, :, None, :]
+    key_states, value_states = repeat_kv(g["kr"], G), repeat_kv(g["vr"], G)
+    scale_key, zero_key = repeat_kv(g["sk"][:, :, None], G), repeat_kv(g["zk"][:, :, None], G)
+    scale_val, zero_val = repeat_kv(g["sv"][:, :, None], G), repeat_kv(g["zv"][:, :, None], G)
+    lut = torch.arange(2, device="cuda", dtype=torch.bfloat16)
+    enc_k, enc_v = repeat_kv(g["ck"], G), repeat_kv(g["cv"], G)
+    w_s = torch.matmul(q, key_states[:, :, :S].transpose(2, 3)) / math.sqrt(128)
+    w_t = torch.matmul(q, key_states[:, :, S:].transpose(2, 3)) / math.sqrt(128)
+    bias_k = torch.sum(scale_key * zero_key * q, dim=-1, keepdim=True) / math.sqrt(128)
+    w_v = cq.fused_kernel(lut, q * scale_key, enc_k) / math.sqrt(128) - bias_k
+    cur_max, cur_min = w_v.amax(dim=(2, 3), keepdim=True), w_v.amin(dim=(2, 3), keepdim=True)
+    w_v = (w_v - cur_min) / (cur_max - cur_min + 1e-8) * ((cur_max - 3) - cur_min) + cur_min
+    p = torch.softmax(torch.cat([w_s, w_v, w_t], dim=-1), dim=-1, dtype=torch.float32).to(q.dtype)
+    out_v = cq.fused_kernel_wv(lut.half(), p[..., S:S + T].half(), enc_v) * scale_val
+    out_v = out_v - scale_val * zero_val * torch.sum(p[..., S:S + T], dim=-1, keepdim=True)
+    out = out_v + torch.matmul(p[..., :S], value_states[:, :, :S]) + torch.matmul(p[..., S + T:], value_states[:, :, S:])
+    fused = ops.decode_attn(g["q"], g["ck"], g["cv"], g["sk"], g["zk"], g["sv"], g["zv"], g["kr"], g["vr"],
+                            sprompt_len=S, bits=bits)
+    err = (out[:, :, 0].float() - fused.float()).abs()
+    assert err.max().item() < 5e-2 and err.mean().item() < 1e-2
+    # and the oracle's restatement of that mixed-precision chain tracks the torch sequence closely
+    chain = O.decode_attention_refchain(c["q"], c["ck"], c["cv"], c["sk"], c["zk"], c["sv"], c["zv"],
+                                        c["kr"], c["vr"], S, bits, "bf16")
+    assert np.abs(chain - to_np(out[:, :, 0])).mean() < 5e-3

@@ -1,0 +1,122 @@
+"""Host-side logic that needs no GPU: the C-ABI library's exports, argument
+validation at the Python boundary, cache bookkeeping, RoPE / GQA helpers."""
+import ctypes
+import math
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    from calibquant_amd import _lib
+    lib = _lib.load()
+    header = open(os.path.join(ROOT, "include", "calibquant_hip.h")).read()
+    declared = set(re.findall(r"\b(cq_[a-z_0-9]+)\s*\(", header))
+    assert declared, "no declarations found"
+    assert declared == set(_lib.SYMBOLS)
+    for name in declared:
+        assert getattr(lib, name) is not None
+    assert lib.cq_version() >= 100
+    assert b"NULL" in lib.cq_strerror(-1) and lib.cq_strerror(0) == b"ok"
+
+
+def test_c_abi_rejects_bad_arguments_without_touching_the_gpu():
+    """Validation happens before any launch, so these calls are safe without a device."""
+    from calibquant_amd import _lib
+    lib = _lib.load()
+    a = _lib.DecodeArgs()
+    assert lib.cq_decode_attn(ctypes.byref(a), None) < 0                  # dtype/shape all zero
+    a.dtype, a.bits, a.D, a.B, a.Hq, a.Hkv, a.T, a.R = 0, 3, 128, 1, 32, 8, 64, 0
+    assert lib.cq_decode_attn(ctypes.byref(a), None) == -7                # 3-bit unsupported
+    a.bits, a.D = 1, 64
+    assert lib.cq_decode_attn(ctypes.byref(a), None) == -7                # head_dim 64 unsupported
+    a.D, a.Hq = 128, 30
+    assert lib.cq_decode_attn(ctypes.byref(a), None) == -2                # Hq not a multiple of Hkv
+    a.Hq, a.T, a.R = 32, 0, 0
+    assert lib.cq_decode_attn(ctypes.byref(a), None) == -2                # nothing to attend to
+    a.T = 64
+    assert lib.cq_decode_attn(ctypes.byref(a), None) == -1                # NULL pointers
+    assert lib.cq_decode_attn_workspace(ctypes.byref(a)) == 0             # fits one unit: no workspace
+    a.T, a.B = 32768, 8
+    ws = lib.cq_decode_attn_workspace(ctypes.byref(a))
+    assert ws > 0 and ws % 4 == 0                                         # chunked path needs partials
+    assert lib.cq_quantize_pack_workspace(64, 3328, 8, 128) == 64 * 8 * 8 * 2 * 128 * 4
+    assert lib.cq_quantize_pack(None, 0, 1, 1, 1, 128, 0, 0, 0, 1, 0.5, None, None, None, None, 0, None) == -1
+    assert lib.cq_encode(None, 3, 1, 128, 1, None, None) == -1
+
+
+def test_ops_refuse_cpu_tensors_and_unsupported_dtypes():
+    from calibquant_amd import ops
+    from calibquant_amd._lib import CalibQuantError
+    x = torch.zeros((1, 4, 1, 128), dtype=torch.bfloat16)
+    with pytest.raises(CalibQuantError, match="GPU"):
+        ops.quantize_pack(x, 1, 0.5)
+    with pytest.raises(CalibQuantError, match="GPU"):
+        ops.decode_attn(torch.zeros((1, 8, 128), dtype=torch.bfloat16), None, None, None, None, None, None, x, x)
+    from calibquant_amd import calibquant
+    with pytest.raises(CalibQuantError):
+        calibquant.quant(x, 1, per_channel=False)
+    with pytest.raises(CalibQuantError):
+        calibquant.quant(x, 4, per_channel=True)
+
+
+def test_reference_constants_and_helpers():
+    from calibquant_amd import calibquant as cq, patch_internvl as pi
+    assert (cq.BITS_KV, cq.SCALE_K, cq.SCALE_V, cq.DEVICE, cq.DATA_TYPE) == (1, 0.5, 0.3, "cuda", torch.float16)
+    assert (pi.BITS_KV, pi.SCALE_K, pi.SCALE_V, pi.SPROMPT_LEN, pi.CHUNK_SIZE, pi.LOW_BITS) == (1, 0.5, 0.3, 41, 1024, True)
+    assert set(pi.ATTN_FORWARD_FUNCTIONS) == {"calibquant", "qjl"}
+    x = torch.arange(2 * 3 * 4 * 5, dtype=torch.float32).reshape(2, 3, 4, 5)
+    assert torch.equal(pi.repeat_kv(x, 3), torch.repeat_interleave(x, 3, dim=1))
+    assert pi.repeat_kv(x, 1) is x
+    # rotary embedding against the textbook complex rotation
+    torch.manual_seed(0)
+    D, N = 8, 6
+    q, k = torch.randn(1, 2, N, D), torch.randn(1, 1, N, D)
+    inv = 1.0 / (10000 ** (torch.arange(0, D, 2).float() / D))
+    ang = torch.outer(torch.arange(N).float(), inv)
+    cos, sin = torch.cat([ang, ang], -1).cos(), torch.cat([ang, ang], -1).sin()
+    pos = torch.arange(N)[None]
+    qe, ke = pi.apply_rotary_pos_emb(q, k, cos, sin, pos)
+    qc = torch.complex(q[..., : D // 2], q[..., D // 2:]) * torch.polar(torch.ones_like(ang), ang)
+    assert torch.allclose(qe, torch.cat([qc.real, qc.imag], -1), atol=1e-6)
+    assert torch.allclose((qe @ ke.transpose(-1, -2))[0, 0].diagonal(), (q @ k.transpose(-1, -2))[0, 0].diagonal(),
+                          atol=1e-4)   # equal positions: rotation cancels in the dot product
+    with pytest.raises(Exception):
+        pi.patch_model(object(), quant_method="qjl")
+
+
+def test_growing_kv_appends_in_place_and_survives_foreign_tensors():
+    from calibquant_amd.kvbuffer import GrowingKV
+    kv = GrowingKV()
+    k0, v0 = torch.randn(2, 3, 5, 4), torch.randn(2, 3, 5, 4)
+    k, v = kv.append(None, k0, v0)
+    assert k.shape == (2, 3, 5, 4) and torch.equal(k, k0)
+    ptr = k.data_ptr()
+    k1, v1 = torch.randn(2, 3, 1, 4), torch.randn(2, 3, 1, 4)
+    k, v = kv.append((k, v), k1, v1)
+    assert k.data_ptr() == ptr and k.shape[2] == 6                      # appended in place
+    assert torch.equal(k[:, :, :5], k0) and torch.equal(k[:, :, 5:], k1) and torch.equal(v[:, :, 5:], v1)
+    foreign = (torch.randn(2, 3, 9, 4), torch.randn(2, 3, 9, 4))
+    k, v = kv.append(foreign, k1, v1)                                    # not ours: copied
+    assert k.shape[2] == 10 and torch.equal(k[:, :, :9], foreign[0]) and torch.equal(k[:, :, 9:], k1)
+    for _ in range(600):                                                 # grow past the capacity
+        k, v = kv.append((k, v), k1, v1)
+    assert k.shape[2] == 610 and torch.equal(k[:, :, :9], foreign[0])
+
+
+def test_internlm2_wqkv_interleave_matches_the_reference_rearrange():
+    """`b q (h gs d) -> b q h gs d` with gs = groups + 2: q heads, then k, then v per kv head."""
+    from einops import rearrange
+    from calibquant_amd.internlm2 import InternLM2Attention, InternLM2Config
+    cfg = InternLM2Config.tiny()
+    att = InternLM2Attention(cfg)
+    x = torch.randn(2, 3, cfg.hidden_size)
+    q, k, v = att.split_qkv(x)
+    qkv = rearrange(att.wqkv(x), "b q (h gs d) -> b q h gs d", gs=2 + att.num_key_value_groups, d=att.head_dim)
+    assert torch.equal(q, rearrange(qkv[..., : att.num_key_value_groups, :], "b q h gs d -> b q (h gs) d"))
+    assert torch.equal(k, qkv[..., -2, :]) and torch.equal(v, qkv[..., -1, :])
