@@ -145,6 +145,74 @@ def cpu_baseline(torch, sets, shape, bits, budget_s=12.0):
                       f"scaled x{B // bs} to the full batch"}
 
 
+def model_leg(torch, batch=64, tiles=13, sys_len=41, text_len=23, new_tokens=128, seed=1234):
+    """InternVL2.5-8B-shaped decode (InternLM2.5-7B language model: 32 layers, hidden 4096, 32/8
+    heads, head_dim 128, vocab 92 553), random-init bf16 weights, synthetic uniform-noise tiles
+    through a stand-in vision tower: tokens/s of `new_tokens` greedy steps at `batch`, prefill
+    excluded, 1-bit KV (patched attention) vs full-precision KV (unpatched) on the same weights."""
+    from calibquant_amd import patch_internvl as pi
+    from calibquant_amd.internlm2 import InternLM2Attention, InternLM2Config, InternVLChatStandIn
+    dev = torch.device("cuda:0")
+    torch.manual_seed(seed)
+    prev = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        with torch.device(dev):
+            model = InternVLChatStandIn(InternLM2Config.internvl2_5_8b()).eval()
+    finally:
+        torch.set_default_dtype(prev)
+    T = tiles * 256
+    N = sys_len + T + text_len
+    ids = torch.randint(0, 90000, (batch, N), device=dev)
+    ids[:, sys_len:sys_len + T] = model.img_context_token_id
+    fp_forward, fp_generate = InternLM2Attention.forward, InternVLChatStandIn.generate
+    res = {"prompt_tokens": N, "image_tokens": T, "new_tokens": new_tokens, "batch": batch}
+
+    def run(tag, patched):
+        stamps = []
+
+        def on_step(i):
+            if i == 0 or i == new_tokens - 1:     # only the two ends of the decode loop synchronise
+                torch.cuda.synchronize()
+                stamps.append(time.perf_counter())
+
+        vis = []
+        with torch.no_grad():
+            # vision features tile-chunked per sample to bound the pixel tensor
+            for b0 in range(0, batch, 8):
+                pix = torch.rand((8 * tiles, 3, 448, 448), device=dev, dtype=torch.bfloat16)
+                vis.append(model.extract_feature(pix))
+            vit = torch.cat(vis, 0)
+            if patched:
+                out = pi.custom_generate(model, pixel_values=torch.empty(0), input_ids=ids, visual_features=vit,
+                                         max_new_tokens=new_tokens, on_step=on_step)
+            else:
+                emb = model.language_model.get_input_embeddings()(ids)
+                emb[ids == model.img_context_token_id] = vit.reshape(-1, emb.shape[-1])
+                out = model.language_model.generate(inputs_embeds=emb, max_new_tokens=new_tokens, on_step=on_step)
+        assert out.shape == (batch, new_tokens)
+        # stamps[0] closes the prefill; the decode steps are the intervals after it
+        dt = stamps[-1] - stamps[0]
+        res[tag + "_decode_tok_s"] = round(batch * (new_tokens - 1) / dt, 1)
+        res[tag + "_ms_per_token_step"] = round(dt / (new_tokens - 1) * 1e3, 3)
+        for layer in model.language_model.model.layers:      # drop the KV state before the next run
+            for name in ("_kv", "_cq_window", "_cq_call", "_cq_stats", "encoded_features_k", "encoded_features_v"):
+                if hasattr(layer.attention, name):
+                    delattr(layer.attention, name)
+        torch.cuda.empty_cache()
+
+    try:
+        run("fp16_kv", False)
+        import contextlib, io
+        with contextlib.redirect_stdout(io.StringIO()):
+            pi.patch_model(model, "calibquant")
+        run("kv_1bit", True)
+    finally:
+        InternLM2Attention.forward, InternVLChatStandIn.generate = fp_forward, fp_generate
+    res["note"] = "eager PyTorch host loop (no graph capture): both legs include per-layer launch overhead"
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -155,6 +223,9 @@ def main():
     ap.add_argument("--sets", type=int, default=4, help="distinct input buffer sets rotated through")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-fp16kv", action="store_true", help="skip the fp16-KV comparison leg")
+    ap.add_argument("--no-model", action="store_true", help="skip the full-model decode tok/s leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch three 256 MiB device copies (known traffic, for scaling profiler byte counters)")
     ap.add_argument("--seed", type=int, default=1234)
     a = ap.parse_args()
     if a.gpus != 1:
@@ -173,6 +244,12 @@ def main():
     sets = build_sets(torch, ops, shape, a.bits, a.sets, a.seed)
     calls = [ops.DecodeCall(s["q"], s["ck"], s["cv"], s["sk"], s["zk"], s["sv"], s["zv"], s["kr"], s["vr"],
                             sprompt_len=S, bits=a.bits) for s in sets]
+    if a.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
     ms = time_calls(torch, calls, a.steps, a.warmup)
     nbytes = algorithmic_bytes(B, Hq, Hkv, D, T, R, a.bits)
     gbps = nbytes / (ms * 1e-3) / 1e9
@@ -207,6 +284,13 @@ def main():
             out["fp16_kv_error"] = repr(e)[:200]
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline(torch, sets, shape, a.bits)
+    if not a.no_model and a.workload == DEFAULT_WORKLOAD and a.bits == 1:
+        del sets, calls
+        torch.cuda.empty_cache()
+        try:
+            out["model_decode"] = model_leg(torch)
+        except Exception as e:  # the model leg must not sink the kernel measurement
+            out["model_decode"] = {"error": repr(e)[:300]}
     print(json.dumps(out))
 
 

@@ -185,6 +185,18 @@ class DecodeCall:
         self.args, self._ref, self._keep, self.out, self.device = a, C.byref(a), keep, out, q.device
         self.workspace_bytes = 0 if ws is None else ws.numel()
 
+    def step(self, q: torch.Tensor, k_res: torch.Tensor, v_res: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        """Re-aim the prepared call at this decode step's query, output and (grown) residual
+        window and launch.  Only pointers, R and the strides change; packed state, dtype, head
+        counts and options stay as prepared.  No validation beyond what the C entry point does."""
+        a = self.args
+        a.q, a.out = q.data_ptr(), out.data_ptr()
+        a.k_res, a.v_res, a.R = k_res.data_ptr(), v_res.data_ptr(), k_res.shape[2]
+        a.res_stride_b, a.res_stride_h, a.res_stride_r = k_res.stride(0), k_res.stride(1), k_res.stride(2)
+        self._step_keep = (q, k_res, v_res, out)
+        self.out = out
+        return self.run()
+
     def run(self) -> torch.Tensor:
         rc = self._lib.cq_decode_attn(self._ref, torch.cuda.current_stream(self.device).cuda_stream)
         if rc:

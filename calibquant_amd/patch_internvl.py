@@ -156,6 +156,7 @@ def forward_internlm2_calibquant(self, hidden_states: torch.Tensor, attention_ma
                                   "the image block of a fresh prompt)")
         if S + T > q_len:
             raise CalibQuantError(f"prompt of {q_len} tokens is shorter than sprompt_len + image tokens = {S + T}")
+        self._cq_call = None
         if T > 0:
             k_img = key_states[:, :, S:S + T, :].transpose(1, 2)      # (B, T, Hkv, D) strided views
             v_img = value_states[:, :, S:S + T, :].transpose(1, 2)
@@ -204,11 +205,21 @@ def forward_internlm2_calibquant(self, hidden_states: torch.Tensor, attention_ma
             raise ValueError(f"Attention mask should be of size {(bsz, 1, q_len, kv_seq_len)}, "
                              f"but is {attention_mask.size()}")
         mask = attention_mask[:, 0, 0, :]
-    stats = self._cq_stats if T > 0 else (None,) * 4
-    out = ops.decode_attn(query_states[:, :, 0, :], self.encoded_features_k if T > 0 else None,
-                          self.encoded_features_v if T > 0 else None, stats[0], stats[1], stats[2], stats[3],
-                          k_res, v_res, sprompt_len=min(S, R), bits=self.bits_k, calibrate=self.normalize,
-                          calib_off_max=CALIB_OFFSET_MAX, calib_off_min=CALIB_OFFSET_MIN, mask=mask)
+    q1 = query_states[:, :, 0, :]
+    call = getattr(self, "_cq_call", None)
+    if (mask is None and call is not None and call.args.B == bsz and call.workspace_bytes == 0
+            and q1.is_contiguous() and call.args.dtype == (0 if q1.dtype == torch.bfloat16 else 1)):
+        # steady state: re-aim the prepared call (same packed state) at this step's tensors
+        out = call.step(q1, k_res, v_res, torch.empty_like(q1))
+    else:
+        stats = self._cq_stats if T > 0 else (None,) * 4
+        call = ops.DecodeCall(q1, self.encoded_features_k if T > 0 else None,
+                              self.encoded_features_v if T > 0 else None, stats[0], stats[1], stats[2], stats[3],
+                              k_res, v_res, sprompt_len=min(S, R), bits=self.bits_k, calibrate=self.normalize,
+                              calib_off_max=CALIB_OFFSET_MAX, calib_off_min=CALIB_OFFSET_MIN, mask=mask)
+        with torch.cuda.device(call.device):
+            out = call.run()
+        self._cq_call = call if mask is None else None
     attn_output = self.wo(out.reshape(bsz, 1, self.hidden_size))
     return attn_output, None, past_key_value
 
