@@ -45,6 +45,17 @@ def algorithmic_bytes(B, Hq, Hkv, D, T, R, bits, elt=2):
     return codes + stats + resid + qo
 
 
+def measured_traffic(workload, bits):
+    """HBM bytes per launch measured with rocprofv3 byte counters (profiles/decode_kernel_traffic.json),
+    or None when that workload has not been profiled."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "decode_kernel_traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(f"{workload}/bits{bits}", {}).get("traffic_bytes")
+    except OSError:
+        return None
+
+
 def build_sets(torch, ops, shape, bits, nsets, seed):
     """Synthetic layer state, generated on the GPU with a seeded device
     generator: K/V ~ N(0,1), four key channels per kv-head scaled by |t3|+1
@@ -271,7 +282,7 @@ def main():
                    "kv_packed_tokens": T, "kv_residual_rows": R, "bits": a.bits, "storage_dtype": "bf16",
                    "buffer_sets": a.sets, "launches_per_step": 1 if calls[0].workspace_bytes == 0 else 3},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": measured_traffic(a.workload, a.bits),
                      "algorithmic_bytes": nbytes},
     }
     if not a.no_fp16kv:
