@@ -100,9 +100,46 @@ __device__ __forceinline__ void store_elem(void* p, int64_t i, float f) {
 // row_bcast:15 = 0x142, row_bcast:31 = 0x143.
 template <int CTRL, int ROW_MASK = 0xf>
 __device__ __forceinline__ float dpp_move(float v, float inactive) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, inactive),
-                                                                  __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf,
-                                                                  false));
+    if constexpr (ROW_MASK == 0xf && CTRL < 0x142) {
+        // every lane has a source: no fill value needed
+        return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+    } else {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, inactive),
+                                                                      __builtin_bit_cast(int, v), CTRL, ROW_MASK,
+                                                                      0xf, false));
+    }
+}
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ int dpp_move_i(int v, int inactive) {
+    if constexpr (ROW_MASK == 0xf && CTRL < 0x142) {
+        return __builtin_amdgcn_mov_dpp(v, CTRL, 0xf, 0xf, true);
+    } else {
+        return __builtin_amdgcn_update_dpp(inactive, v, CTRL, ROW_MASK, 0xf, false);
+    }
+}
+
+// Order-preserving map between floats and signed integers (an involution): integer
+// max / min then orders like the float one, and fuses with the cross-lane modifiers.
+__device__ __forceinline__ int float_key(float f) {
+    const int i = __builtin_bit_cast(int, f);
+    return i ^ ((i >> 31) & 0x7fffffff);
+}
+__device__ __forceinline__ float key_float(int k) { return __builtin_bit_cast(float, k ^ ((k >> 31) & 0x7fffffff)); }
+
+// max over aligned groups of 16 lanes / the whole wave, on integer keys
+__device__ __forceinline__ int row_max_key(int v) {
+    constexpr int lo = static_cast<int>(0x80000000u);
+    v = max(v, dpp_move_i<0xB1>(v, lo));
+    v = max(v, dpp_move_i<0x4E>(v, lo));
+    v = max(v, dpp_move_i<0x141>(v, lo));
+    return max(v, dpp_move_i<0x140>(v, lo));
+}
+__device__ __forceinline__ int wave_max_key(int v) {
+    constexpr int lo = static_cast<int>(0x80000000u);
+    v = row_max_key(v);
+    v = max(v, dpp_move_i<0x142, 0xa>(v, lo));
+    v = max(v, dpp_move_i<0x143, 0xc>(v, lo));
+    return __builtin_amdgcn_readlane(v, 63);
 }
 
 struct OpMin { __device__ __forceinline__ float operator()(float a, float b) const { return fminf(a, b); } };
@@ -129,7 +166,7 @@ template <typename Op> __device__ __forceinline__ float wave_reduce(float v, Op 
     v = op(v, dpp_move<0x143, 0xc>(v, id));
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
-__device__ __forceinline__ float wave_max(float v) { return wave_reduce(v, OpMax(), -INFINITY); }
+__device__ __forceinline__ float wave_max(float v) { return key_float(wave_max_key(float_key(v))); }
 __device__ __forceinline__ float wave_min(float v) { return wave_reduce(v, OpMin(), INFINITY); }
 __device__ __forceinline__ float wave_sum(float v) { return wave_reduce(v, OpSum(), 0.0f); }
 

@@ -90,7 +90,7 @@ template <int BITS, int HPB> struct Lay {
     static constexpr int F_QSZ = F_QF + HPB * kD;             // HPB*kD
     static constexpr int F_QRAW = F_QSZ + HPB * kD;           // HPB*kD raw 16-bit q
     static constexpr int F_RED = F_QRAW + HPB * kD / 2;       // kNW*HPB
-    static constexpr int F_STAT = F_RED + kNW * HPB;          // 8*HPB: per-head softmax state
+    static constexpr int F_STAT = F_RED + 2 * kNW * HPB;      // 8*HPB: per-head softmax state
     static constexpr int F_VSZ = F_STAT + 8 * HPB;            // 2*kD: value scale, zero-point
     static constexpr int F_NIB = F_VSZ + 2 * kD;              // NB*32*HPB: nibble tables
     static constexpr int F_SRES = F_NIB + NB * 32 * HPB;      // kResTile*HPB
@@ -126,6 +126,26 @@ __device__ __forceinline__ void block_reduce(float* v, float* red, Op op, float 
         float x = (lane < kNW) ? red[lane * HPB + h] : identity;
         x = row_reduce(x, op, identity);   // lanes 0..15 hold the partials
         v[h] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, x)));
+    }
+    __syncthreads();
+}
+
+// Block-wide maximum of N values (integer keys, see float_key); result wave-uniform.
+template <int N>
+__device__ __forceinline__ void block_max(float* v, float* red) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    int* redi = reinterpret_cast<int*>(red);
+#pragma unroll
+    for (int h = 0; h < N; ++h) {
+        const int x = wave_max_key(float_key(v[h]));
+        if (lane == 0) redi[w * N + h] = x;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int h = 0; h < N; ++h) {
+        int x = (lane < kNW) ? redi[lane * N + h] : static_cast<int>(0x80000000u);
+        x = row_max_key(x);
+        v[h] = key_float(__builtin_amdgcn_readfirstlane(x));
     }
     __syncthreads();
 }
@@ -420,9 +440,13 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
             for (int r = 0; r < L::KR; ++r) token_logits(tb + tid + r * kNT, kc[r]);
         }
     }
-    if (n > 0) {
-        block_reduce<HPB>(mn, red, OpMin(), INFINITY);
-        block_reduce<HPB>(mx, red, OpMax(), -INFINITY);
+    if (n > 0) {   // one reduction for both: max of (-min, max)
+        float mm2[2 * HPB];
+#pragma unroll
+        for (int h = 0; h < HPB; ++h) { mm2[h] = -mn[h]; mm2[HPB + h] = mx[h]; }
+        block_max<2 * HPB>(mm2, red);
+#pragma unroll
+        for (int h = 0; h < HPB; ++h) { mn[h] = -mm2[h]; mx[h] = mm2[HPB + h]; }
     }
 
     if constexpr (MINMAX_ONLY) {
@@ -457,10 +481,10 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     const int wi = static_cast<int>(w[q]);
-                    const uint32_t x0 = __builtin_amdgcn_update_dpp(0, wi, 0x00, 0xf, 0xf, false);
-                    const uint32_t x1 = __builtin_amdgcn_update_dpp(0, wi, 0x55, 0xf, 0xf, false);
-                    const uint32_t x2 = __builtin_amdgcn_update_dpp(0, wi, 0xAA, 0xf, 0xf, false);
-                    const uint32_t x3 = __builtin_amdgcn_update_dpp(0, wi, 0xFF, 0xf, 0xf, false);
+                    const uint32_t x0 = __builtin_amdgcn_mov_dpp(wi, 0x00, 0xf, 0xf, true);
+                    const uint32_t x1 = __builtin_amdgcn_mov_dpp(wi, 0x55, 0xf, 0xf, true);
+                    const uint32_t x2 = __builtin_amdgcn_mov_dpp(wi, 0xAA, 0xf, 0xf, true);
+                    const uint32_t x3 = __builtin_amdgcn_mov_dpp(wi, 0xFF, 0xf, 0xf, true);
                     const uint32_t lo = __builtin_amdgcn_perm(x1, x0, sel_pair);
                     const uint32_t hi = __builtin_amdgcn_perm(x3, x2, sel_pair);
                     const uint32_t t4 = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
@@ -513,7 +537,7 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                     }
                     logits[tt] = w;
                 }
-                block_reduce<HPB>(lm, red, OpMax(), -INFINITY);
+                block_max<HPB>(lm, red);
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) { m_img[h] = lm[h]; slope[h] = 1.0f; tmin[h] = 0.f; mn[h] = 0.f; }
             } else {
@@ -523,6 +547,14 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
             float ls[HPB];
 #pragma unroll
             for (int h = 0; h < HPB; ++h) ls[h] = 0.f;
+            // e = exp(x - M) with x = (w - mn) * slope + tmin, as exp2((w - mn) * ea + ec)
+            float ea[HPB], ec[HPB];
+#pragma unroll
+            for (int h = 0; h < HPB; ++h) {
+                const bool dead = (m_img[h] == -INFINITY);   // every position masked out
+                ea[h] = dead ? 0.f : slope[h] * kLog2e;
+                ec[h] = dead ? -INFINITY : (tmin[h] - m_img[h]) * kLog2e;
+            }
             using HWv = Words<L::HW>;
             for (int tt = tid; tt < npad; tt += kNT) {
                 float e[4] = {0.f, 0.f, 0.f, 0.f};
@@ -530,8 +562,7 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                     const V w = logits[tt];
 #pragma unroll
                     for (int h = 0; h < HPB; ++h) {
-                        const float x = (w.v[h] - mn[h]) * slope[h] + tmin[h];
-                        e[h] = (m_img[h] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((x - m_img[h]) * kLog2e);
+                        e[h] = __builtin_amdgcn_exp2f((w.v[h] - mn[h]) * ea[h] + ec[h]);
                         ls[h] += e[h];
                     }
                 }
