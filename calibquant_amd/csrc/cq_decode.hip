@@ -173,6 +173,16 @@ template <> __device__ __forceinline__ float dot2<FP16>(uint32_t a, uint32_t b, 
 
 template <int N> struct alignas(N * 4) Words { uint32_t w[N]; };
 
+// N dwords at an absolute LDS byte address (N-dword aligned): one ds_read of that width.
+template <int N> __device__ __forceinline__ Words<N> lds_words(uint32_t addr) {
+    typedef uint32_t VT __attribute__((ext_vector_type(N)));
+    const VT v = *(const __attribute__((address_space(3))) VT*)(static_cast<uintptr_t>(addr));
+    Words<N> r;
+#pragma unroll
+    for (int k = 0; k < N; ++k) r.w[k] = v[k];
+    return r;
+}
+
 __device__ __forceinline__ uint32_t pack_f16(float a, float b) {
     f16x2_t h = {static_cast<_Float16>(a), static_cast<_Float16>(b)};   // round to nearest even
     return __builtin_bit_cast(uint32_t, h);
@@ -240,12 +250,6 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                                : static_cast<const uint4*>(g.q);
     const U4* cvp4 = reinterpret_cast<const U4*>(cvp);
     const int last_u = has_img ? n * NB / 16 - 1 : 0;   // last valid 16-byte unit of either stream
-    uint4 kc[L::KR][BITS];
-#pragma unroll
-    for (int r = 0; r < L::KR; ++r) {
-#pragma unroll
-        for (int i = 0; i < BITS; ++i) kc[r][i] = ckp[min((tid + r * kNT) * BITS + i, last_u)];
-    }
     // residual tile: K slice (row = tid/8, 16 elements) and V slices (two rows, 8 elements)
     const int l8 = tid & 7, krow = tid >> 3;
     // residual V: lane = (8-element slice ds, row slot): the slot's two low bits sit in the
@@ -273,6 +277,13 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
     if constexpr (!MINMAX_ONLY) {
         load_res_k(0, rk);
         load_res_v(0, rv);
+    }
+    uint4 kc[L::KR][BITS];
+#pragma unroll
+    for (int r = 0; r < L::KR; ++r) {   // first half now, second half once the residual phase is done
+#pragma unroll
+        for (int i = 0; i < BITS; ++i)
+            if (r * BITS + i < kPF / 2) kc[r][i] = ckp[min((tid + r * kNT) * BITS + i, last_u)];
     }
 
     // ---- phase 0: q, per-bit weights ---------------------------------------------------
@@ -303,13 +314,123 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
     }
     __syncthreads();
 
+    float* stat = fx + L::F_STAT;   // [alpha | m_res | l_res | m_img | l_img][HPB]
+    float o_res = 0.f;
+    if constexpr (!MINMAX_ONLY) {
+        // ---- phase 1: full-precision residual rows, online softmax.  Runs first: its rows
+        // were requested first, and the packed K rows keep streaming in meanwhile.
+#pragma unroll
+        for (int h = 0; h < HPB; ++h) {
+            if (tid == h) {
+                stat[HPB + h] = -INFINITY;
+                stat[2 * HPB + h] = 0.f;
+            }
+        }
+        if (do_res) {
+            float m_run = -INFINITY, l_run = 0.f;
+            float* sres = fx + L::F_SRES;
+            float* pres = fx + L::F_PRES;
+            // raw 16-bit q, [head][kD], read per head as two 16-byte LDS loads
+            const uint4* q128 = reinterpret_cast<const uint4*>(fx + L::F_QRAW);
+            float accv[8][HPB];
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+#pragma unroll
+                for (int h = 0; h < HPB; ++h) accv[k][h] = 0.f;
+            const float* mk = g.mask ? g.mask + b * g.mask_sb : nullptr;
+
+            for (int r0 = 0; r0 < g.R; r0 += kResTile) {
+                const bool more = r0 + kResTile < g.R;
+                const int r = r0 + krow;
+                float dot[HPB];
+#pragma unroll
+                for (int h = 0; h < HPB; ++h) {
+                    const uint4 qa = q128[h * (kD / 8) + l8];
+                    const uint4 qb = q128[h * (kD / 8) + 8 + l8];
+                    float a = 0.f;
+                    a = dot2<DT>(qa.x, rk[0].x, a); a = dot2<DT>(qa.y, rk[0].y, a);
+                    a = dot2<DT>(qa.z, rk[0].z, a); a = dot2<DT>(qa.w, rk[0].w, a);
+                    a = dot2<DT>(qb.x, rk[1].x, a); a = dot2<DT>(qb.y, rk[1].y, a);
+                    a = dot2<DT>(qb.z, rk[1].z, a); a = dot2<DT>(qb.w, rk[1].w, a);
+                    dot[h] = oct_reduce(a, OpSum(), 0.f) * inv_sqrt_d;
+                }
+                if (more) load_res_k(r0 + kResTile, rk);   // next tile's K slice, in place
+                if (l8 == 0) {
+                    float mv = 0.f;
+                    if (mk && r < g.R) mv = mk[r < g.S ? r : g.T + r];
+#pragma unroll
+                    for (int h = 0; h < HPB; ++h) sres[krow * HPB + h] = (r < g.R) ? dot[h] + mv : -INFINITY;
+                }
+                __syncthreads();
+                if (wv < HPB) {   // wave h keeps the running softmax state of head h
+                    const int h = wv;
+                    const float s0 = sres[lane * HPB + h];
+                    const float s1 = sres[(lane + 64) * HPB + h];
+                    const float mnew = fmaxf(m_run, wave_max(fmaxf(s0, s1)));
+                    const bool dead = (mnew == -INFINITY);
+                    const float p0 = dead ? 0.f : __expf(s0 - mnew);
+                    const float p1 = dead ? 0.f : __expf(s1 - mnew);
+                    const float al = dead ? 1.0f : __expf(m_run - mnew);
+                    l_run = l_run * al + wave_sum(p0 + p1);
+                    m_run = mnew;
+                    pres[lane * HPB + h] = p0;
+                    pres[(lane + 64) * HPB + h] = p1;
+                    if (lane == 0) { stat[h] = al; stat[HPB + h] = m_run; stat[2 * HPB + h] = l_run; }
+                }
+                __syncthreads();
+                float alpha[HPB];
+#pragma unroll
+                for (int h = 0; h < HPB; ++h) alpha[h] = stat[h];
+#pragma unroll
+                for (int rep = 0; rep < 2; ++rep) {
+                    const int rr = rslot + rep * (kResTile / 2);
+                    float f[8];
+                    unpack8<DT>(rv[rep], f);
+                    const V p = reinterpret_cast<const V*>(pres)[rr];   // 0 for rows past R
+#pragma unroll
+                    for (int k = 0; k < 8; ++k)
+#pragma unroll
+                        for (int h = 0; h < HPB; ++h)
+                            accv[k][h] = ((rep == 0 && r0 > 0) ? accv[k][h] * alpha[h] : accv[k][h]) + p.v[h] * f[k];
+                }
+                if (more) load_res_v(r0 + kResTile, rv);   // next tile's V slices, in place
+            }
+            // fold the row slots: 4 per wave (lane bits 4,5), then the waves
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+#pragma unroll
+                for (int h = 0; h < HPB; ++h) accv[k][h] = quad_reduce(accv[k][h], OpSum(), 0.f);
+            __syncthreads();
+            float* red2 = reinterpret_cast<float*>(regA);  // [wave][kD][HPB]
+            if ((lane & 3) == 0) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+#pragma unroll
+                    for (int h = 0; h < HPB; ++h) red2[(wv * kD + ds * 8 + k) * HPB + h] = accv[k][h];
+            }
+            __syncthreads();
+            if (tid < HPB * kD) {
+                const int h = tid / kD, d = tid % kD;
+#pragma unroll
+                for (int w = 0; w < kNW; ++w) o_res += red2[(w * kD + d) * HPB + h];
+            }
+        }
+
+    }
+
+#pragma unroll
+    for (int r = 0; r < L::KR; ++r) {
+#pragma unroll
+        for (int i = 0; i < BITS; ++i)
+            if (r * BITS + i >= kPF / 2) kc[r][i] = ckp[min((tid + r * kNT) * BITS + i, last_u)];
+    }
     float mn[HPB], mx[HPB];
 #pragma unroll
     for (int h = 0; h < HPB; ++h) { mn[h] = INFINITY; mx[h] = -INFINITY; }
     U4 vc[kPF];   // first block of packed V rows, requested as the packed K registers free up
 
     if (n > 0) {
-        // ---- phase 1: byte table = high-nibble table + low-nibble table ----------------
+        // ---- phase 2: byte table = high-nibble table + low-nibble table ----------------
         // nibble tables: entry (j, half, v) = sum of the per-bit weights v selects; the
         // zero-point sum of the byte position is folded into the high half.
         V* nib = reinterpret_cast<V*>(fx + L::F_NIB);   // [half*16 + value][byte position]
@@ -349,7 +470,7 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
         }
         __syncthreads();
 
-        // ---- phase 2: logits of the chunk ------------------------------------------------
+        // ---- phase 3: logits of the chunk ------------------------------------------------
         // Lane l walks the byte positions in the order k ^ (l mod NB): in every step the
         // lanes that the LDS serves together read NB distinct positions of the
         // position-fastest table, i.e. distinct banks whatever the byte values are.  The
@@ -500,7 +621,7 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                 }
             }
 
-            // ---- phase 3: calibration + exp ---------------------------------------------
+            // ---- phase 4: calibration + exp ---------------------------------------------
             if (g.nsplit > 1) {
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) {
@@ -576,7 +697,7 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
 #pragma unroll
             for (int h = 0; h < HPB; ++h) l_img[h] = ls[h];
 
-            // ---- phase 4: packed V ----------------------------------------------------------
+            // ---- phase 5: packed V ----------------------------------------------------------
             // lane = (byte column j, slice c of its 8 bit lanes); a wave pass covers TPW tokens
             unsigned char* wtab = regA + wv * (L::GPW * 16 * L::ESZH);
             const int j = lane / L::GPW, cs = lane % L::GPW;
@@ -593,13 +714,25 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) acc[m][h] = 0.f;
             const float one = g.one;
-            // bit lane m of the byte is bit 7 - m; entry offset = sum_i bit(token i) * ESZH * 2^i
-            uint32_t shr[L::MPL];
+            // Bit lane m of a byte is bit 7 - m; table offset = sum_i bit(token i) * ESZH * 2^i.
+            // The lane's MPL bit lanes sit in one nibble: the dword is shifted by 4 * (m < 4) once,
+            // each lane masks its bit in place (value 2^s per byte) and the dot-product
+            // multiplier carries the 2^-s: ESZH * 2^i >> s stays integral for s <= 3, ESZH = 8;
+            // with 4-byte entries the multiplier is kept whole and s = 0 (bit moved down first).
+            constexpr bool kInPlace = (L::ESZH == 8);
+            const uint32_t nib_shift = (cs * L::MPL < 4) ? 4u : 0u;
+            uint32_t bmask[L::MPL], bmult[L::MPL], bshr[L::MPL];
 #pragma unroll
-            for (int m = 0; m < L::MPL; ++m) shr[m] = 7 - (cs * L::MPL + m);
-            constexpr uint32_t kMult = L::ESZH * 0x08040201u;
+            for (int m = 0; m < L::MPL; ++m) {
+                const uint32_t sft = 3 - ((cs * L::MPL + m) & 3);   // bit position inside the nibble
+                bmask[m] = kInPlace ? (0x01010101u << sft) : 0x01010101u;
+                bmult[m] = kInPlace ? ((L::ESZH * 0x08040201u) >> sft) & 0x7f7f7f7fu : L::ESZH * 0x08040201u;
+                bshr[m] = kInPlace ? 0u : sft;
+            }
             using WG = Words<L::GPW>;   // the GPW dwords of one (unit, column)
-            const uint32_t wtab_addr = static_cast<uint32_t>(wtab - smem);   // byte offset in LDS
+            // absolute LDS address of the wave's tables (the dot product's addend)
+            const uint32_t wtab_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+                (__attribute__((address_space(3))) unsigned char*)wtab));
 
             for (int vs0 = 0; vs0 < npad; vs0 += L::VSUB) {
                 const int vn = min(L::VSUB, npad - vs0);
@@ -638,11 +771,12 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
 #pragma unroll
                     for (int gq = 0; gq < L::GPW; ++gq) {
                         const uint32_t tbase = wtab_addr + static_cast<uint32_t>(gq * 16 * L::ESZH);
+                        const uint32_t wsh = cw.w[gq] >> nib_shift;
 #pragma unroll
                         for (int m = 0; m < L::MPL; ++m) {
-                            const uint32_t bits = (cw.w[gq] >> shr[m]) & 0x01010101u;
-                            const uint32_t off = __builtin_amdgcn_udot4(bits, kMult, tbase, false);
-                            const HWv e = *reinterpret_cast<const HWv*>(smem + off);
+                            const uint32_t bits = (kInPlace ? wsh : (wsh >> bshr[m])) & bmask[m];
+                            const uint32_t off = __builtin_amdgcn_udot4(bits, bmult[m], tbase, false);
+                            const HWv e = lds_words<L::HW>(off);
 #pragma unroll
                             for (int h = 0; h < HPB; ++h) {
                                 const f16x2_t pr = __builtin_bit_cast(f16x2_t, e.w[h >> 1]);
@@ -686,108 +820,13 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
             __syncthreads();
         }
 
-        // ---- phase 5: full-precision residual rows, online softmax ----------------------
-        float* stat = fx + L::F_STAT;   // [alpha | m_res | l_res | m_img | l_img][HPB]
 #pragma unroll
         for (int h = 0; h < HPB; ++h) {
             if (tid == h) {
-                stat[HPB + h] = -INFINITY;
-                stat[2 * HPB + h] = 0.f;
                 stat[3 * HPB + h] = m_img[h];
                 stat[4 * HPB + h] = l_img[h];
             }
         }
-        float o_res = 0.f;
-        if (do_res) {
-            float m_run = -INFINITY, l_run = 0.f;
-            float* sres = fx + L::F_SRES;
-            float* pres = fx + L::F_PRES;
-            // raw 16-bit q, [head][kD], read per head as two 16-byte LDS loads
-            const uint4* q128 = reinterpret_cast<const uint4*>(fx + L::F_QRAW);
-            float accv[8][HPB];
-#pragma unroll
-            for (int k = 0; k < 8; ++k)
-#pragma unroll
-                for (int h = 0; h < HPB; ++h) accv[k][h] = 0.f;
-            const float* mk = g.mask ? g.mask + b * g.mask_sb : nullptr;
-
-            for (int r0 = 0; r0 < g.R; r0 += kResTile) {
-                const bool more = r0 + kResTile < g.R;
-                const int r = r0 + krow;
-                float dot[HPB];
-#pragma unroll
-                for (int h = 0; h < HPB; ++h) {
-                    const uint4 qa = q128[h * (kD / 8) + l8];
-                    const uint4 qb = q128[h * (kD / 8) + 8 + l8];
-                    float a = 0.f;
-                    a = dot2<DT>(qa.x, rk[0].x, a); a = dot2<DT>(qa.y, rk[0].y, a);
-                    a = dot2<DT>(qa.z, rk[0].z, a); a = dot2<DT>(qa.w, rk[0].w, a);
-                    a = dot2<DT>(qb.x, rk[1].x, a); a = dot2<DT>(qb.y, rk[1].y, a);
-                    a = dot2<DT>(qb.z, rk[1].z, a); a = dot2<DT>(qb.w, rk[1].w, a);
-                    dot[h] = oct_reduce(a, OpSum(), 0.f) * inv_sqrt_d;
-                }
-                if (more) load_res_k(r0 + kResTile, rk);   // next tile's K slice, in place
-                if (l8 == 0) {
-                    float mv = 0.f;
-                    if (mk && r < g.R) mv = mk[r < g.S ? r : g.T + r];
-#pragma unroll
-                    for (int h = 0; h < HPB; ++h) sres[krow * HPB + h] = (r < g.R) ? dot[h] + mv : -INFINITY;
-                }
-                __syncthreads();
-                if (wv < HPB) {   // wave h keeps the running softmax state of head h
-                    const int h = wv;
-                    const float s0 = sres[lane * HPB + h];
-                    const float s1 = sres[(lane + 64) * HPB + h];
-                    const float mnew = fmaxf(m_run, wave_max(fmaxf(s0, s1)));
-                    const bool dead = (mnew == -INFINITY);
-                    const float p0 = dead ? 0.f : __expf(s0 - mnew);
-                    const float p1 = dead ? 0.f : __expf(s1 - mnew);
-                    const float al = dead ? 1.0f : __expf(m_run - mnew);
-                    l_run = l_run * al + wave_sum(p0 + p1);
-                    m_run = mnew;
-                    pres[lane * HPB + h] = p0;
-                    pres[(lane + 64) * HPB + h] = p1;
-                    if (lane == 0) { stat[h] = al; stat[HPB + h] = m_run; stat[2 * HPB + h] = l_run; }
-                }
-                __syncthreads();
-                float alpha[HPB];
-#pragma unroll
-                for (int h = 0; h < HPB; ++h) alpha[h] = stat[h];
-#pragma unroll
-                for (int rep = 0; rep < 2; ++rep) {
-                    const int rr = rslot + rep * (kResTile / 2);
-                    float f[8];
-                    unpack8<DT>(rv[rep], f);
-                    const V p = reinterpret_cast<const V*>(pres)[rr];   // 0 for rows past R
-#pragma unroll
-                    for (int k = 0; k < 8; ++k)
-#pragma unroll
-                        for (int h = 0; h < HPB; ++h)
-                            accv[k][h] = ((rep == 0 && r0 > 0) ? accv[k][h] * alpha[h] : accv[k][h]) + p.v[h] * f[k];
-                }
-                if (more) load_res_v(r0 + kResTile, rv);   // next tile's V slices, in place
-            }
-            // fold the row slots: 4 per wave (lane bits 4,5), then the waves
-#pragma unroll
-            for (int k = 0; k < 8; ++k)
-#pragma unroll
-                for (int h = 0; h < HPB; ++h) accv[k][h] = quad_reduce(accv[k][h], OpSum(), 0.f);
-            __syncthreads();
-            float* red2 = reinterpret_cast<float*>(regA);  // [wave][kD][HPB]
-            if ((lane & 3) == 0) {
-#pragma unroll
-                for (int k = 0; k < 8; ++k)
-#pragma unroll
-                    for (int h = 0; h < HPB; ++h) red2[(wv * kD + ds * 8 + k) * HPB + h] = accv[k][h];
-            }
-            __syncthreads();
-            if (tid < HPB * kD) {
-                const int h = tid / kD, d = tid % kD;
-#pragma unroll
-                for (int w = 0; w < kNW; ++w) o_res += red2[(w * kD + d) * HPB + h];
-            }
-        }
-
         // ---- phase 6: merge / write ---------------------------------------------------------
         __syncthreads();
         if (tid < HPB * kD) {
