@@ -486,6 +486,14 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
 #pragma unroll
         for (int k = 0; k < NB; ++k) pofs[k] = (k ^ skew) * L::ESZ;
         const unsigned char* ktab_b = regA;
+        // With 256-byte table rows the address of a look-up is two bytes side by side, the
+        // byte value above the position offset: one byte permute builds it from the row word
+        // and a word holding four position offsets.
+        constexpr bool kPermAddr = (NB * L::ESZ == 256);
+        uint32_t pofs4[NB / 4];
+#pragma unroll
+        for (int i = 0; i < NB / 4; ++i)
+            pofs4[i] = pofs[4 * i] | (pofs[4 * i + 1] << 8) | (pofs[4 * i + 2] << 16) | (pofs[4 * i + 3] << 24);
         auto token_logits = [&](int tt, const uint4* c) {
             if (tt < n) {
                 uint32_t w[NW32];
@@ -510,8 +518,14 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                 V part[6];
 #pragma unroll
                 for (int k = 0; k < NB; ++k) {
-                    const uint32_t byte = (wds[k >> 2] >> (8 * (k & 3))) & 0xffu;
-                    V cur = *reinterpret_cast<const V*>(ktab_b + byte * (NB * L::ESZ) + pofs[k]);
+                    V cur;
+                    if constexpr (kPermAddr) {
+                        const uint32_t sel = static_cast<uint32_t>(k & 3) | (static_cast<uint32_t>(4 + (k & 3)) << 8) | 0x0c0c0000u;
+                        cur = *reinterpret_cast<const V*>(ktab_b + __builtin_amdgcn_perm(wds[k >> 2], pofs4[k >> 2], sel));
+                    } else {
+                        const uint32_t byte = (wds[k >> 2] >> (8 * (k & 3))) & 0xffu;
+                        cur = *reinterpret_cast<const V*>(ktab_b + byte * (NB * L::ESZ) + pofs[k]);
+                    }
 #pragma unroll
                     for (int l = 0; l < 6; ++l) {
                         if ((k >> l) & 1) {
@@ -768,6 +782,10 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                     __builtin_amdgcn_wave_barrier();
                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                    // The GPW entries a bit lane picks in this pass (each at most 4) are first
+                    // added as packed fp16 pairs, pairwise; one mixed-precision FMA per head then
+                    // moves the sum into the fp32 accumulator.
+                    f16x2_t pk[L::MPL][L::GPW][L::HW];
 #pragma unroll
                     for (int gq = 0; gq < L::GPW; ++gq) {
                         const uint32_t tbase = wtab_addr + static_cast<uint32_t>(gq * 16 * L::ESZH);
@@ -778,11 +796,22 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                             const uint32_t off = __builtin_amdgcn_udot4(bits, bmult[m], tbase, false);
                             const HWv e = lds_words<L::HW>(off);
 #pragma unroll
-                            for (int h = 0; h < HPB; ++h) {
-                                const f16x2_t pr = __builtin_bit_cast(f16x2_t, e.w[h >> 1]);
-                                const _Float16 hv = (h & 1) ? pr.y : pr.x;
-                                acc[m][h] = __builtin_fmaf(static_cast<float>(hv), one, acc[m][h]);
-                            }
+                            for (int k = 0; k < L::HW; ++k) pk[m][gq][k] = __builtin_bit_cast(f16x2_t, e.w[k]);
+                        }
+                    }
+#pragma unroll
+                    for (int m = 0; m < L::MPL; ++m) {
+#pragma unroll
+                        for (int st = 1; st < L::GPW; st *= 2)
+#pragma unroll
+                            for (int gq = 0; gq + st < L::GPW; gq += 2 * st)
+#pragma unroll
+                                for (int k = 0; k < L::HW; ++k) pk[m][gq][k] += pk[m][gq + st][k];
+#pragma unroll
+                        for (int h = 0; h < HPB; ++h) {
+                            const f16x2_t pr = pk[m][0][h >> 1];
+                            const _Float16 hv = (h & 1) ? pr.y : pr.x;
+                            acc[m][h] = __builtin_fmaf(static_cast<float>(hv), one, acc[m][h]);
                         }
                     }
                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
