@@ -37,6 +37,7 @@ class DecodeArgs(C.Structure):
         ("T", C.c_int), ("R", C.c_int), ("sprompt_len", C.c_int), ("bits", C.c_int),
         ("calibrate", C.c_int), ("calib_off_max", C.c_float), ("calib_off_min", C.c_float),
         ("force_splits", C.c_int),
+        ("r_dev", C.c_void_p),
     ]
 
 

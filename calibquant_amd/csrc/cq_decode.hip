@@ -56,6 +56,7 @@ struct DecodeGeom {
     const float* mask;
     int64_t mask_sb;
     void* out;
+    const int32_t* r_dev;   // optional: residual row count read at run time (R is then the capacity)
     float* mm;    // [B][Hq][nsplit][2] chunk logit min / max
     float* part;  // [B][Hq][nx][kD + 2] partials (m, l, acc)
     int B, Hq, Hkv, T, R, S;
@@ -218,7 +219,8 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
     const int64_t bh = static_cast<int64_t>(b) * g.Hkv + hkv;
 
     const bool img_unit = split < g.nsplit && g.T > 0;
-    const bool do_res = !MINMAX_ONLY && g.R > 0 && (g.nsplit == 1 || split == g.nsplit);
+    const int R = g.r_dev ? min(*g.r_dev, g.R) : g.R;   // rows in the residual window
+    const bool do_res = !MINMAX_ONLY && R > 0 && (g.nsplit == 1 || split == g.nsplit);
     const int t0 = img_unit ? split * g.chunk : 0;
     const int n = img_unit ? min(g.T, t0 + g.chunk) - t0 : 0;
     const int npad = (n + L::TPW - 1) / L::TPW * L::TPW;
@@ -259,7 +261,7 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                                 : static_cast<const uint16_t*>(g.q);
     const uint16_t* vbp = do_res ? static_cast<const uint16_t*>(g.vres) + b * g.rs_b + hkv * g.rs_h
                                  : static_cast<const uint16_t*>(g.q);
-    const int last_r = do_res ? g.R - 1 : 0;
+    const int last_r = do_res ? R - 1 : 0;
     const int64_t rs_r = do_res ? g.rs_r : 0;
     uint4 rk[2], rv[2];
     auto load_res_k = [&](int r0, uint4* k2) {   // rows past R re-read row R-1 (their logit is masked)
@@ -339,8 +341,8 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                 for (int h = 0; h < HPB; ++h) accv[k][h] = 0.f;
             const float* mk = g.mask ? g.mask + b * g.mask_sb : nullptr;
 
-            for (int r0 = 0; r0 < g.R; r0 += kResTile) {
-                const bool more = r0 + kResTile < g.R;
+            for (int r0 = 0; r0 < R; r0 += kResTile) {
+                const bool more = r0 + kResTile < R;
                 const int r = r0 + krow;
                 float dot[HPB];
 #pragma unroll
@@ -357,9 +359,9 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                 if (more) load_res_k(r0 + kResTile, rk);   // next tile's K slice, in place
                 if (l8 == 0) {
                     float mv = 0.f;
-                    if (mk && r < g.R) mv = mk[r < g.S ? r : g.T + r];
+                    if (mk && r < R) mv = mk[r < g.S ? r : g.T + r];
 #pragma unroll
-                    for (int h = 0; h < HPB; ++h) sres[krow * HPB + h] = (r < g.R) ? dot[h] + mv : -INFINITY;
+                    for (int h = 0; h < HPB; ++h) sres[krow * HPB + h] = (r < R) ? dot[h] + mv : -INFINITY;
                 }
                 __syncthreads();
                 if (wv < HPB) {   // wave h keeps the running softmax state of head h
@@ -1023,6 +1025,8 @@ int cq_decode_attn(const cq_decode_args* a, cq_stream_t stream) {
     if (a->T > 0 && (!a->codes_k || !a->codes_v || !a->k_scale || !a->k_zero || !a->v_scale || !a->v_zero))
         return CQ_ERR_NULL;
     if (a->R > 0 && (!a->k_res || !a->v_res)) return CQ_ERR_NULL;
+    if (a->r_dev && a->mask) return CQ_ERR_UNSUPPORTED;   // the mask's length would have to follow the count
+    if (a->r_dev && (reinterpret_cast<uintptr_t>(a->r_dev) & 3)) return CQ_ERR_ALIGN;
     if (a->T > 0 && (!cq::aligned16(a->codes_k) || !cq::aligned16(a->codes_v))) return CQ_ERR_ALIGN;
     if (a->R > 0 && (!cq::aligned16(a->k_res) || !cq::aligned16(a->v_res) || (a->res_stride_b % 8) ||
                      (a->res_stride_h % 8) || (a->res_stride_r % 8)))
@@ -1036,6 +1040,7 @@ int cq_decode_attn(const cq_decode_args* a, cq_stream_t stream) {
     g.kres = a->k_res; g.vres = a->v_res;
     g.rs_b = a->res_stride_b; g.rs_h = a->res_stride_h; g.rs_r = a->res_stride_r;
     g.mask = a->mask; g.mask_sb = a->mask_stride_b;
+    g.r_dev = a->r_dev;
     g.out = a->out;
     g.mm = static_cast<float*>(a->workspace);
     g.part = need ? reinterpret_cast<float*>(static_cast<char*>(a->workspace) + p.ws_mm) : nullptr;

@@ -122,7 +122,7 @@ class DecodeCall:
 
     def __init__(self, q, codes_k, codes_v, k_scale, k_zero, v_scale, v_zero, k_res, v_res,
                  sprompt_len=0, bits=1, calibrate=True, calib_off_max=-3.0, calib_off_min=0.0,
-                 mask=None, out=None, force_splits=0):
+                 mask=None, out=None, force_splits=0, r_dev=None):
         _need_gpu(q, "q")
         dt = _storage_dtype(q, "q")
         if q.dim() != 3:
@@ -177,6 +177,16 @@ class DecodeCall:
         a.calibrate = int(bool(calibrate))
         a.calib_off_max, a.calib_off_min = float(calib_off_max), float(calib_off_min)
         a.force_splits = int(force_splits)
+        if r_dev is not None:
+            # residual row count read on the device at run time; k_res / v_res are then the
+            # whole window buffers (capacity rows) and R is that capacity
+            _need_gpu(r_dev, "r_dev")
+            if r_dev.dtype != torch.int32 or r_dev.numel() != 1:
+                raise _lib.CalibQuantError("r_dev must be a single int32 on the GPU")
+            if mask is not None:
+                raise _lib.CalibQuantError("r_dev and mask cannot be combined")
+            a.r_dev = r_dev.data_ptr()
+            keep.append(r_dev)
         self._lib = _lib.load()
         ws = _workspace(self._lib.cq_decode_attn_workspace(C.byref(a)), q.device)
         if ws is not None:
@@ -211,13 +221,15 @@ def decode_attn(q: torch.Tensor, codes_k: Optional[torch.Tensor], codes_v: Optio
                 sprompt_len: int = 0, bits: int = 1, calibrate: bool = True,
                 calib_off_max: float = -3.0, calib_off_min: float = 0.0,
                 mask: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
-                force_splits: int = 0) -> torch.Tensor:
+                force_splits: int = 0, r_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One decode-attention step over packed image K/V plus the fp residual window.
 
     q (B, Hq, D); codes_* uint8 (B, Hkv, T, D*bits/8); *_scale, *_zero (B, Hkv, D);
     k_res, v_res (B, Hkv, R, D) (any b/h/r strides); mask optional additive
-    (B, S + T + R - S) over the [sys | image | text] order.  Returns (B, Hq, D)."""
+    (B, S + T + R - S) over the [sys | image | text] order.  `r_dev` (int32 GPU scalar): the
+    number of valid rows of k_res / v_res, read on the device when the launch runs.
+    Returns (B, Hq, D)."""
     call = DecodeCall(q, codes_k, codes_v, k_scale, k_zero, v_scale, v_zero, k_res, v_res,
-                      sprompt_len, bits, calibrate, calib_off_max, calib_off_min, mask, out, force_splits)
+                      sprompt_len, bits, calibrate, calib_off_max, calib_off_min, mask, out, force_splits, r_dev)
     with torch.cuda.device(call.device):
         return call.run()

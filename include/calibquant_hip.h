@@ -143,6 +143,15 @@ typedef struct cq_decode_args {
     float calib_off_max;   /* reference: -3 */
     float calib_off_min;   /* reference:  0 */
     int force_splits;   /* 0 = choose; >0 = split the T axis into this many chunks */
+    /* Optional: device pointer to the number of residual rows.  When not NULL
+     * the kernels read the row count from it at run time (0 <= *r_dev <= R,
+     * sprompt_len <= *r_dev) and R above is only the capacity of the window
+     * buffers.  A caller that replays a recorded launch (a HIP graph of a
+     * decode step) grows the window this way without changing the launch:
+     * the reference re-reads the window's length from the tensor shape on
+     * every step (patch_internvl.py:246-251,265-266), which a recorded
+     * launch cannot.  Must be NULL when a mask is given. */
+    const int32_t* r_dev;
 } cq_decode_args;
 
 size_t cq_decode_attn_workspace(const cq_decode_args* args);

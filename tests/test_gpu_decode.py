@@ -112,6 +112,31 @@ def test_decode_attn_residual_only_and_strided_cache(ops):
     _check(to_np(out2), _oracle(c, 41, 1))
 
 
+@pytest.mark.parametrize("splits", [0, 3])
+def test_decode_attn_row_count_read_on_device(ops, splits):
+    """Window buffers of fixed capacity, the number of valid rows in a device
+    scalar: the same prepared launch follows the window as it grows (what a
+    recorded decode step needs).  Rows past the count hold garbage."""
+    B, Hq, Hkv, T, R, S = 2, 32, 8, 1500, 150, 41
+    c = make_case(B, Hq, Hkv, 128, T, R, 1, "bf16", seed=21)
+    g = case_to_gpu(c, "bf16")
+    cap = 192
+    kbuf = torch.full((B, Hkv, cap, 128), 1e4, dtype=torch.bfloat16, device="cuda")
+    vbuf = torch.full_like(kbuf, -1e4)
+    kbuf[:, :, :R] = g["kr"]
+    vbuf[:, :, :R] = g["vr"]
+    r_dev = torch.zeros(1, dtype=torch.int32, device="cuda")
+    call = ops.DecodeCall(g["q"], g["ck"], g["cv"], g["sk"], g["zk"], g["sv"], g["zv"], kbuf, vbuf,
+                          sprompt_len=S, bits=1, force_splits=splits, r_dev=r_dev)
+    for rows in (60, 150, 129):          # grow, then shrink: only the scalar changes
+        r_dev.fill_(rows)
+        got = to_np(call.run())
+        torch.cuda.synchronize()
+        want = O.decode_attention(c["q"], c["ck"], c["cv"], c["sk"], c["zk"], c["sv"], c["zv"],
+                                  c["kr"][:, :, :rows], c["vr"][:, :, :rows], S, 1)
+        _check(got, want)
+
+
 @pytest.mark.parametrize("bits", [1, 2])
 @pytest.mark.parametrize("splits", [2, 5])
 def test_decode_attn_split_path_matches_fused_path(ops, bits, splits):
