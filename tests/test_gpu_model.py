@@ -121,3 +121,67 @@ def test_patch_model_and_custom_generate_end_to_end():
         assert torch.equal(out, out2)
     finally:
         InternLM2Attention.forward, InternVLChatStandIn.generate = fp_forward, fp_generate
+
+
+def _prefill(m, ids, pix=None):
+    """Prompt embeddings (image features spliced in) -> last-position logits and the per-layer cache."""
+    lm = m.language_model
+    emb = lm.get_input_embeddings()(ids)
+    if pix is not None:
+        vit = m.extract_feature(pix)
+        emb = emb.clone()
+        emb[ids == m.img_context_token_id] = vit.reshape(-1, emb.shape[-1]).to(emb.dtype)
+    B, N = ids.shape
+    pos = torch.arange(N, device=ids.device)[None].expand(B, N)
+    return lm.forward_step(emb, pos, None)
+
+
+@pytest.mark.parametrize("quantized", [True, False])
+def test_static_decoder_graph_replays_equal_eager_steps(quantized):
+    """The recorded decode step, replayed per token, produces the tokens of the same step run
+    eagerly, and its first step agrees with the model's own eager step."""
+    from calibquant_amd import patch_internvl as pi
+    from calibquant_amd.graph_decode import StaticDecoder
+    from calibquant_amd.internlm2 import InternLM2Attention, InternVLChatStandIn
+    fp_forward, fp_generate = InternLM2Attention.forward, InternVLChatStandIn.generate
+    m = _tiny_model(seed=5)
+    lm = m.language_model
+    B, S, tiles, txt, NEW = 2, 41, 2, 9, 12
+    T = tiles * 256
+    ids = torch.randint(0, 500, (B, S + T + txt), device="cuda")
+    ids[:, S:S + T] = m.img_context_token_id
+    pix = torch.rand(B * tiles, 3, 448, 448, device="cuda", dtype=torch.bfloat16)
+    N = ids.shape[1]
+    try:
+        with torch.no_grad():
+            if quantized:
+                pi.patch_model(m, "calibquant")
+                for layer in lm.model.layers:
+                    layer.attention.image_token_num = T
+            runs = []
+            for use_graph in (False, True):
+                logits, past = _prefill(m, ids, pix)
+                first = logits[:, -1].argmax(-1)
+                dec = StaticDecoder(lm, past, N, NEW)
+                toks = dec.generate(first, NEW, use_graph=use_graph)
+                torch.cuda.synchronize()
+                assert (dec.graph is not None) == use_graph
+                runs.append(toks)
+            assert torch.equal(runs[0], runs[1])
+            # first decode step against the model's eager forward_step (different norm kernel,
+            # same arithmetic up to rounding)
+            logits, past = _prefill(m, ids, pix)
+            first = logits[:, -1].argmax(-1)
+            dec = StaticDecoder(lm, past, N, 2)
+            dec.tok.copy_(first)
+            x = lm.get_input_embeddings()(first)[:, None]
+            pos1 = torch.full((B, 1), N, device="cuda", dtype=torch.long)
+            want, _ = lm.forward_step(x, pos1, past)
+            lay = lm.model.layers
+            got_tok = dec.step().clone()
+            assert runs[0][:, 1].tolist() == got_tok.tolist()
+            # the eager model's choice has (near-)maximal logit under the static step as well
+            w = want[:, -1].float()
+            assert ((w.max(-1).values - w.gather(1, got_tok[:, None])[:, 0]) < 0.15).all()
+    finally:
+        InternLM2Attention.forward, InternVLChatStandIn.generate = fp_forward, fp_generate
