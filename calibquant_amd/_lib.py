@@ -16,7 +16,7 @@ SYMBOLS = (
     "cq_version", "cq_strerror", "cq_last_hip_error",
     "cq_quantize_pack_workspace", "cq_quantize_pack", "cq_quant", "cq_encode",
     "cq_lut_vecmat_qk", "cq_lut_vecmat_pv",
-    "cq_decode_attn_workspace", "cq_decode_attn",
+    "cq_decode_attn_workspace", "cq_decode_attn", "cq_rope_append",
 )
 
 
@@ -80,6 +80,8 @@ def load() -> C.CDLL:
     lib.cq_decode_attn_workspace.argtypes = [C.POINTER(DecodeArgs)]
     lib.cq_decode_attn.restype = i
     lib.cq_decode_attn.argtypes = [C.POINTER(DecodeArgs), vp]
+    lib.cq_rope_append.restype = i
+    lib.cq_rope_append.argtypes = [vp, i, i, i, i, i, vp, vp, i64, vp, i64, vp, vp, vp, i64, i64, i64, i, vp, vp]
     _lib = lib
     return lib
 

@@ -14,7 +14,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIBPATH = os.path.join(LIBDIR, "libcalibquant_hip.so")
-SOURCES = ["cq_core.hip", "cq_quantize.hip", "cq_lutvecmat.hip", "cq_decode.hip"]
+SOURCES = ["cq_core.hip", "cq_quantize.hip", "cq_lutvecmat.hip", "cq_decode.hip", "cq_rope.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

@@ -28,15 +28,10 @@ from ._lib import CalibQuantError
 from .patch_internvl import CALIB_OFFSET_MAX, CALIB_OFFSET_MIN
 
 
-def _rotate_half(x):
-    h = x.shape[-1] // 2
-    return torch.cat((-x[..., h:], x[..., :h]), dim=-1)
-
-
 class _LayerState:
     """Fixed-address decode state of one attention module."""
 
-    def __init__(self, att, past, capacity: int, r_len: torch.Tensor, quantized: bool):
+    def __init__(self, att, past, capacity: int, r_len: torch.Tensor, quantized: bool, cos, sin, pos, row):
         k_old, v_old = past
         B, Hkv, R0, D = k_old.shape
         self.quantized = quantized
@@ -49,6 +44,10 @@ class _LayerState:
         Hq = att.num_heads
         self.q = torch.empty((B, Hq, D), dtype=k_old.dtype, device=k_old.device)
         self.out = torch.empty_like(self.q)
+        # fused projection output of the step's token, and the launch that splits it, applies
+        # the rotary embedding and appends the key / value row to the window
+        self.qkv = torch.empty((B, (Hq + 2 * Hkv) * D), dtype=k_old.dtype, device=k_old.device)
+        self.rope = ops.RopeAppendCall(self.qkv, cos, sin, pos, self.q, self.kbuf, self.vbuf, row)
         self.call = None
         if quantized:
             T = att.image_token_num
@@ -85,10 +84,11 @@ class StaticDecoder:
         self.r_idx = torch.full((1,), R0, dtype=torch.long, device=dev)
         self.pos = torch.full((self.B, 1), prompt_len, dtype=torch.long, device=dev)
         self.tok = torch.zeros((self.B,), dtype=torch.long, device=dev)
-        self.state: List[_LayerState] = [
-            _LayerState(l.attention, past[i], self.capacity, self.r_len, self.quantized) for i, l in enumerate(layers)]
         cos, sin = att0.rotary_emb(k0, seq_len=prompt_len + max_new_tokens + 1)
         self.cos, self.sin = cos.contiguous(), sin.contiguous()
+        self.state: List[_LayerState] = [
+            _LayerState(l.attention, past[i], self.capacity, self.r_len, self.quantized, self.cos, self.sin,
+                        self.pos, self.r_idx) for i, l in enumerate(layers)]
         self.col = torch.arange(self.capacity, device=dev)
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.steps_left = max_new_tokens
@@ -97,28 +97,19 @@ class StaticDecoder:
     def _step(self):
         lm = self.lm
         x = lm.get_input_embeddings()(self.tok)[:, None]                      # (B, 1, hidden)
-        cos = self.cos[self.pos].unsqueeze(1)                                 # (B, 1, 1, D)
-        sin = self.sin[self.pos].unsqueeze(1)
         for layer, st in zip(lm.model.layers, self.state):
             att = layer.attention
-            B, G, D, Hq = self.B, att.num_key_value_groups, att.head_dim, att.num_heads
-            Hkv = Hq // G
+            B = self.B
             h = F.rms_norm(x, (x.shape[-1],), layer.attention_norm.weight, layer.attention_norm.eps)
-            qkv = att.wqkv(h).view(B, 1, Hkv, 2 + G, D)
-            q = qkv[..., :G, :].reshape(B, 1, Hq, D).transpose(1, 2)          # (B, Hq, 1, D)
-            k = qkv[..., -2, :].transpose(1, 2)                               # (B, Hkv, 1, D)
-            v = qkv[..., -1, :].transpose(1, 2)
-            q = q * cos + _rotate_half(q) * sin
-            k = k * cos + _rotate_half(k) * sin
-            st.kbuf.index_copy_(2, self.r_idx, k)
-            st.vbuf.index_copy_(2, self.r_idx, v)
+            torch.matmul(h.view(B, -1), att.wqkv.weight.t(), out=st.qkv)
+            st.rope.run()            # st.q <- rotated query heads; window row r_idx <- rotated key, value
             if st.quantized:
-                st.q.copy_(q[:, :, 0, :])
                 st.call.run()
                 o = st.out
             else:
                 keep = (self.col < self.r_len.to(torch.long))[None, None, None, :]
-                o = F.scaled_dot_product_attention(q, st.kbuf, st.vbuf, attn_mask=keep, enable_gqa=True)
+                o = F.scaled_dot_product_attention(st.q[:, :, None, :], st.kbuf, st.vbuf, attn_mask=keep,
+                                                   enable_gqa=True)
             x = x + att.wo(o.reshape(B, 1, att.hidden_size))
             h = F.rms_norm(x, (x.shape[-1],), layer.ffn_norm.weight, layer.ffn_norm.eps)
             x = x + layer.feed_forward(h)

@@ -233,3 +233,40 @@ def decode_attn(q: torch.Tensor, codes_k: Optional[torch.Tensor], codes_v: Optio
                       sprompt_len, bits, calibrate, calib_off_max, calib_off_min, mask, out, force_splits, r_dev)
     with torch.cuda.device(call.device):
         return call.run()
+
+
+class RopeAppendCall:
+    """A prepared `cq_rope_append` launch over fixed buffers: the token's fused projection output
+    `qkv` (B, 1, (Hq + 2 Hkv) * D) or (B, Hkv, Hq/Hkv + 2, D), rotary tables (rows, D), device
+    position ids `pos` (B,) or (B, 1) int64, output query `q_out` (B, Hq, D), the window buffers
+    (B, Hkv, capacity, D) and the device int64 `row` that names the window row to fill."""
+
+    def __init__(self, qkv, cos, sin, pos, q_out, k_win, v_win, row):
+        for t, name in ((qkv, "qkv"), (cos, "cos"), (sin, "sin"), (pos, "pos"), (q_out, "q_out"),
+                        (k_win, "k_win"), (v_win, "v_win"), (row, "row")):
+            _need_gpu(t, name)
+        dt = _storage_dtype(qkv, "qkv")
+        B, Hq, D = q_out.shape
+        Hkv, cap = k_win.shape[1], k_win.shape[2]
+        for t in (cos, sin, q_out, k_win, v_win):
+            if t.dtype != qkv.dtype:
+                raise _lib.CalibQuantError("rope_append: all floating tensors must share the storage dtype")
+        if not (qkv.is_contiguous() and cos.is_contiguous() and sin.is_contiguous() and q_out.is_contiguous()):
+            raise _lib.CalibQuantError("rope_append: qkv, cos, sin and q_out must be contiguous")
+        if qkv.numel() != B * (Hq + 2 * Hkv) * D or cos.shape != sin.shape or cos.shape[-1] != D:
+            raise _lib.CalibQuantError("rope_append: shape mismatch")
+        if k_win.stride() != v_win.stride() or k_win.stride(3) != 1 or k_win.shape != v_win.shape:
+            raise _lib.CalibQuantError("rope_append: window buffers must share shape and strides")
+        if pos.dtype != torch.int64 or row.dtype != torch.int64 or pos.numel() != B or row.numel() != 1:
+            raise _lib.CalibQuantError("rope_append: pos (B int64) / row (1 int64) expected")
+        self._lib = _lib.load()
+        self._keep = (qkv, cos, sin, pos, q_out, k_win, v_win, row)
+        self.device = qkv.device
+        self._args = (qkv.data_ptr(), dt, B, Hq, Hkv, D, cos.data_ptr(), sin.data_ptr(), cos.shape[0],
+                      pos.data_ptr(), pos.reshape(B).stride(0), q_out.data_ptr(), k_win.data_ptr(), v_win.data_ptr(),
+                      k_win.stride(0), k_win.stride(1), k_win.stride(2), cap, row.data_ptr())
+
+    def run(self) -> None:
+        rc = self._lib.cq_rope_append(*self._args, torch.cuda.current_stream(self.device).cuda_stream)
+        if rc:
+            _lib.check(rc, "cq_rope_append")

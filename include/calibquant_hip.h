@@ -157,6 +157,26 @@ typedef struct cq_decode_args {
 size_t cq_decode_attn_workspace(const cq_decode_args* args);
 int cq_decode_attn(const cq_decode_args* args, cq_stream_t stream);
 
+/* ------------------------------------------------------------------------
+ * Decode-step glue, one launch per layer and token: the (h gs d) split of
+ * the fused wqkv output (patch_internvl.py:219-234), rotary embedding of the
+ * query and key heads (patch_internvl.py:119-138, 258-260; x*cos +
+ * rotate_half(x)*sin, rounded to the storage dtype after every op as the
+ * chain of torch ops does) and the append of the new key / value row to the
+ * full-precision window (the reference's torch.cat, patch_internvl.py:264-266).
+ * qkv: (B, Hkv, Hq/Hkv + 2, D) contiguous, one token per sample; cos_table,
+ * sin_table: (table_rows, D) in the storage dtype; pos: device int64,
+ * sample b at pos[b*pos_stride] (clamped to the table); q_out: (B, Hq, D)
+ * contiguous; k_win, v_win: (B, Hkv, capacity, D) through element strides;
+ * row_dev: device int64, the window row that receives the new key / value
+ * (nothing is written if it is outside [0, capacity)).  Position and row are
+ * read on the device, so a recorded launch can be replayed. */
+int cq_rope_append(const void* qkv, int dtype, int B, int Hq, int Hkv, int D,
+                   const void* cos_table, const void* sin_table, int64_t table_rows,
+                   const int64_t* pos, int64_t pos_stride, void* q_out,
+                   void* k_win, void* v_win, int64_t win_stride_b, int64_t win_stride_h,
+                   int64_t win_stride_r, int capacity, const int64_t* row_dev, cq_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -88,3 +88,40 @@ def test_unfused_reference_sequence_agrees_with_the_fused_kernel(cq):
     chain = O.decode_attention_refchain(c["q"], c["ck"], c["cv"], c["sk"], c["zk"], c["sv"], c["zv"],
                                         c["kr"], c["vr"], S, bits, "bf16")
     assert np.abs(chain - to_np(out[:, :, 0])).mean() < 5e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("heads", [(32, 8), (48, 8), (8, 8)])
+def test_rope_append_equals_the_torch_op_chain_bit_for_bit(dtype, heads):
+    """Split of the fused projection, rotary embedding and window append in one launch against
+    the reference's chain of torch ops (patch_internvl.py:119-138, 219-234, 264-266)."""
+    from calibquant_amd import ops, patch_internvl as pi
+    Hq, Hkv = heads
+    G, D, B, cap, rows = Hq // Hkv, 128, 3, 40, 300
+    torch.manual_seed(4)
+    qkv = torch.randn(B, 1, (Hq + 2 * Hkv) * D, device="cuda").to(dtype)
+    t = torch.arange(rows, device="cuda", dtype=torch.float32)
+    inv = 1.0 / (1e6 ** (torch.arange(0, D, 2, device="cuda").float() / D))
+    emb = torch.cat([torch.outer(t, inv)] * 2, dim=-1)
+    cos, sin = emb.cos().to(dtype), emb.sin().to(dtype)
+    pos = torch.tensor([[7], [250], [0]], device="cuda", dtype=torch.long)
+    row = torch.tensor([17], device="cuda", dtype=torch.long)
+    kwin = torch.zeros(B, Hkv, cap, D, device="cuda", dtype=dtype)
+    vwin = torch.zeros_like(kwin)
+    q_out = torch.empty(B, Hq, D, device="cuda", dtype=dtype)
+    ops.RopeAppendCall(qkv, cos, sin, pos, q_out, kwin, vwin, row).run()
+    torch.cuda.synchronize()
+    v5 = qkv.view(B, 1, Hkv, 2 + G, D)
+    q = v5[..., :G, :].reshape(B, 1, Hq, D).transpose(1, 2)
+    k = v5[..., -2, :].transpose(1, 2)
+    v = v5[..., -1, :].transpose(1, 2)
+    qr, kr = pi.apply_rotary_pos_emb(q, k, cos, sin, pos)
+    assert torch.equal(q_out, qr[:, :, 0])
+    assert torch.equal(kwin[:, :, 17], kr[:, :, 0]) and torch.equal(vwin[:, :, 17], v[:, :, 0])
+    kwin[:, :, 17] = 0
+    vwin[:, :, 17] = 0
+    assert not kwin.any() and not vwin.any()          # nothing else was written
+    row.fill_(cap)                                     # a row outside the window: keys / values are dropped
+    ops.RopeAppendCall(qkv, cos, sin, pos, q_out, kwin, vwin, row).run()
+    torch.cuda.synchronize()
+    assert not kwin.any() and not vwin.any()
