@@ -5,11 +5,18 @@
 // work is three launches on one stream:
 //   1. partial min/max per (batch, head, token chunk, channel)  - reads x once
 //   2. statistics: combine the chunks, run the storage-dtype op chain
-//   3. emit: re-read x (L2 / Infinity Cache resident at prefill sizes),
-//      produce the codes and pack them
+//      and, per channel, the input thresholds at which the code steps up
+//   3. emit: re-read x, compare against the thresholds, pack the codes
 // Every arithmetic step that the reference performs as a separate torch op on
 // a 16-bit tensor is rounded to that dtype here (rnd<DT>), and divisions are
 // IEEE (__fdiv_rn); contraction is off so no multiply-add is fused.
+//
+// For a positive finite scale the code is a non-decreasing step function of the
+// input (division by a positive number, adding a constant, rounding, clamping are
+// all monotone), so it is fixed by L thresholds per channel: the smallest storage
+// value that yields code k.  The statistics kernel finds them by bisection over
+// the ordered 16-bit values, evaluating the exact op chain, and the emit kernel
+// only compares - the per-element IEEE division would otherwise bound the pass.
 #include "cq_common.h"
 
 #pragma clang fp contract(off)
@@ -80,13 +87,36 @@ __global__ __launch_bounds__(kQThreads) void minmax_partial_kernel(const uint16_
     }
 }
 
+// One element of calibquant.py:36: round(clamp(x / scale + zero_point, 0, L)).
+// Returns the rounded value; NaN stays NaN (the reference's LUT search then
+// finds no match and yields index 0).
+template <typename DT>
+__device__ __forceinline__ float quant_value(float x, float s, float zp, float levels) {
+    float y = rnd<DT>(__fdiv_rn(x, s));
+    y = rnd<DT>(y + zp);
+    if (y != y) return y;
+    y = fminf(fmaxf(y, 0.0f), levels);
+    return rintf(y);
+}
+
+// Monotone map between the 16-bit storage patterns and integers: order of the keys =
+// order of the values (-inf lowest, +inf highest; NaN patterns lie outside [kKeyLo, kKeyHi]).
+template <typename DT> struct Keys;
+template <> struct Keys<BF16> { static constexpr int lo = -0x7f80, hi = 0x7f80; };
+template <> struct Keys<FP16> { static constexpr int lo = -0x7c00, hi = 0x7c00; };
+template <typename DT>
+__device__ __forceinline__ float key_value(int key) {   // key >= 0: pattern key; key < 0: sign bit + (-key)
+    const uint32_t bits = key >= 0 ? static_cast<uint32_t>(key) : (0x8000u | static_cast<uint32_t>(-key));
+    return Cvt<DT>::to_float(bits);
+}
+
 // ---- 2. statistics ---------------------------------------------------------
 // grid (B*H), D threads.  The op chain of calibquant.py:27-34 with one
 // rounding per op; `tensor / python_scalar` is a multiply by the fp32
 // reciprocal, as torch's device kernel does.
 template <typename DT>
 __global__ void stats_kernel(const float* __restrict__ part, QuantGeom g, float clip, float levels,
-                             uint16_t* __restrict__ scale, uint16_t* __restrict__ zero) {
+                             uint16_t* __restrict__ scale, uint16_t* __restrict__ zero, float* __restrict__ thr) {
     const int bh = blockIdx.x;
     const int d = threadIdx.x;
     if (d >= g.D) return;
@@ -104,18 +134,34 @@ __global__ void stats_kernel(const float* __restrict__ part, QuantGeom g, float 
     const float zp = rnd<DT>(__fdiv_rn(-x_min, s));
     scale[static_cast<int64_t>(bh) * g.D + d] = static_cast<uint16_t>(Cvt<DT>::from_float(s));
     zero[static_cast<int64_t>(bh) * g.D + d] = static_cast<uint16_t>(Cvt<DT>::from_float(zp));
-}
 
-// One element of calibquant.py:36: round(clamp(x / scale + zero_point, 0, L)).
-// Returns the rounded value; NaN stays NaN (the reference's LUT search then
-// finds no match and yields index 0).
-template <typename DT>
-__device__ __forceinline__ float quant_value(float x, float s, float zp, float levels) {
-    float y = rnd<DT>(__fdiv_rn(x, s));
-    y = rnd<DT>(y + zp);
-    if (y != y) return y;
-    y = fminf(fmaxf(y, 0.0f), levels);
-    return rintf(y);
+    // thresholds thr[k-1] = smallest storage value whose code is >= k (k = 1..L), kept as
+    // [k][channel].  NaN in thr[0]: the step-function argument does not hold for this channel
+    // (scale not positive and finite, or zero-point NaN) and emit evaluates the chain itself.
+    float* o = thr + static_cast<int64_t>(bh) * 3 * g.D + d;
+    const bool monotone = s > 0.0f && s < INFINITY && zp == zp;
+    const int nlev = static_cast<int>(levels);
+    for (int k = 1; k <= 3; ++k) {
+        float t = NAN;   // no value reaches code k
+        if (monotone && k <= nlev) {
+            int lo = Keys<DT>::lo, hi = Keys<DT>::hi;   // invariant: code(lo) < k (or lo is the floor), answer in (lo, hi]
+            if (quant_value<DT>(key_value<DT>(hi), s, zp, levels) >= static_cast<float>(k)) {
+                if (quant_value<DT>(key_value<DT>(lo), s, zp, levels) >= static_cast<float>(k)) {
+                    hi = lo;
+                } else {
+                    while (hi - lo > 1) {
+                        const int mid = lo + (hi - lo) / 2;
+                        if (quant_value<DT>(key_value<DT>(mid), s, zp, levels) >= static_cast<float>(k)) hi = mid;
+                        else lo = mid;
+                    }
+                }
+                t = key_value<DT>(hi);
+            }
+        }
+        if (k == 1 && !monotone) t = NAN;
+        o[(k - 1) * g.D] = t;
+    }
+    if (!monotone) o[g.D] = 1.0f;   // thr[1] distinguishes "not monotone" (non-NaN) from "code 1 unreachable" (NaN)
 }
 
 // ---- 3. emit -----------------------------------------------------------------
@@ -125,6 +171,7 @@ template <typename DT, int BITS, bool XQ>
 __global__ __launch_bounds__(kQThreads) void emit_kernel(const uint16_t* __restrict__ x, QuantGeom g,
                                                         const uint16_t* __restrict__ scale,
                                                         const uint16_t* __restrict__ zero,
+                                                        const float* __restrict__ thr,
                                                         uint8_t* __restrict__ codes, uint16_t* __restrict__ xq) {
     const int lpr = g.D >> 3;
     const int rows_per_iter = kQThreads / lpr;
@@ -144,14 +191,39 @@ __global__ __launch_bounds__(kQThreads) void emit_kernel(const uint16_t* __restr
         unpack8<DT>(sv, s);
         unpack8<DT>(zv, zp);
     }
+    // thresholds of this lane's 8 channels; `slow`: a channel without the step-function property
+    float th[BITS == 1 ? 1 : 3][8];
+    bool slow = false;
+    {
+        const float* tp = thr + bh * 3 * g.D + lane * 8;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+#pragma unroll
+            for (int k = 0; k < (BITS == 1 ? 1 : 3); ++k) th[k][i] = tp[k * g.D + i];
+            const float t1 = tp[g.D + i];
+            slow = slow || (th[0][i] != th[0][i] && t1 == t1);
+        }
+    }
     const int nb = g.D * BITS / 8;  // bytes per packed row
     for (int t = t0 + row; t < t1; t += rows_per_iter) {
         uint4 v = *reinterpret_cast<const uint4*>(base + t * g.st);
         float f[8];
         unpack8<DT>(v, f);
         float qv[8];
+        if (!slow) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) qv[i] = quant_value<DT>(f[i], s[i], zp[i], levels);
+            for (int i = 0; i < 8; ++i) {
+                qv[i] = (f[i] >= th[0][i]) ? 1.0f : 0.0f;
+                if constexpr (BITS == 2) {
+                    qv[i] += (f[i] >= th[1][i]) ? 1.0f : 0.0f;
+                    qv[i] += (f[i] >= th[2][i]) ? 1.0f : 0.0f;
+                }
+                if constexpr (XQ) qv[i] = (f[i] != f[i]) ? f[i] : qv[i];   // a NaN input stays NaN in x_q
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) qv[i] = quant_value<DT>(f[i], s[i], zp[i], levels);
+        }
         if constexpr (XQ) {
             uint32_t w[4];
 #pragma unroll
@@ -188,19 +260,20 @@ static int run_quant(const void* x, QuantGeom g, int bits, float clip, uint8_t* 
     hipLaunchKernelGGL(minmax_partial_kernel<DT>, grid, dim3(kQThreads), 0, st, xp, g, ws);
     CQ_LAUNCH_CHECK();
     const float levels = static_cast<float>((1 << bits) - 1);
-    hipLaunchKernelGGL(stats_kernel<DT>, dim3(g.B * g.H), dim3(g.D), 0, st, ws, g, clip, levels, sp, zp);
+    float* thr = ws + static_cast<size_t>(g.B) * g.H * g.nchunk * 2 * g.D;
+    hipLaunchKernelGGL(stats_kernel<DT>, dim3(g.B * g.H), dim3(g.D), 0, st, ws, g, clip, levels, sp, zp, thr);
     CQ_LAUNCH_CHECK();
     uint16_t* xqp = static_cast<uint16_t*>(xq);
     if (xq) {
         if (bits == 1)
-            hipLaunchKernelGGL((emit_kernel<DT, 1, true>), grid, dim3(kQThreads), 0, st, xp, g, sp, zp, codes, xqp);
+            hipLaunchKernelGGL((emit_kernel<DT, 1, true>), grid, dim3(kQThreads), 0, st, xp, g, sp, zp, thr, codes, xqp);
         else
-            hipLaunchKernelGGL((emit_kernel<DT, 2, true>), grid, dim3(kQThreads), 0, st, xp, g, sp, zp, codes, xqp);
+            hipLaunchKernelGGL((emit_kernel<DT, 2, true>), grid, dim3(kQThreads), 0, st, xp, g, sp, zp, thr, codes, xqp);
     } else {
         if (bits == 1)
-            hipLaunchKernelGGL((emit_kernel<DT, 1, false>), grid, dim3(kQThreads), 0, st, xp, g, sp, zp, codes, xqp);
+            hipLaunchKernelGGL((emit_kernel<DT, 1, false>), grid, dim3(kQThreads), 0, st, xp, g, sp, zp, thr, codes, xqp);
         else
-            hipLaunchKernelGGL((emit_kernel<DT, 2, false>), grid, dim3(kQThreads), 0, st, xp, g, sp, zp, codes, xqp);
+            hipLaunchKernelGGL((emit_kernel<DT, 2, false>), grid, dim3(kQThreads), 0, st, xp, g, sp, zp, thr, codes, xqp);
     }
     CQ_LAUNCH_CHECK();
     return CQ_OK;
@@ -280,7 +353,8 @@ extern "C" {
 
 size_t cq_quantize_pack_workspace(int B, int T, int H, int D) {
     if (B < 1 || T < 1 || H < 1 || D < 1) return 0;
-    return static_cast<size_t>(B) * H * cq::pick_chunks(B, T, H) * 2 * D * sizeof(float);
+    // partial min / max per chunk, then three thresholds per channel
+    return static_cast<size_t>(B) * H * (static_cast<size_t>(cq::pick_chunks(B, T, H)) * 2 + 3) * D * sizeof(float);
 }
 
 int cq_quantize_pack(const void* x, int dtype, int B, int T, int H, int D, int64_t stride_b, int64_t stride_t,
