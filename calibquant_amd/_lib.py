@@ -16,7 +16,7 @@ SYMBOLS = (
     "cq_version", "cq_strerror", "cq_last_hip_error",
     "cq_quantize_pack_workspace", "cq_quantize_pack", "cq_quant", "cq_encode",
     "cq_lut_vecmat_qk", "cq_lut_vecmat_pv",
-    "cq_decode_attn_workspace", "cq_decode_attn", "cq_rope_append",
+    "cq_decode_attn_workspace", "cq_decode_attn", "cq_rope_append", "cq_quantize_pack_token",
 )
 
 
@@ -38,6 +38,7 @@ class DecodeArgs(C.Structure):
         ("calibrate", C.c_int), ("calib_off_max", C.c_float), ("calib_off_min", C.c_float),
         ("force_splits", C.c_int),
         ("r_dev", C.c_void_p),
+        ("v_mode", C.c_int),
     ]
 
 
@@ -80,6 +81,8 @@ def load() -> C.CDLL:
     lib.cq_decode_attn_workspace.argtypes = [C.POINTER(DecodeArgs)]
     lib.cq_decode_attn.restype = i
     lib.cq_decode_attn.argtypes = [C.POINTER(DecodeArgs), vp]
+    lib.cq_quantize_pack_token.restype = i
+    lib.cq_quantize_pack_token.argtypes = [vp, i, i, i, i, i, i64, i64, i64, i, i, vp, vp, vp, vp]
     lib.cq_rope_append.restype = i
     lib.cq_rope_append.argtypes = [vp, i, i, i, i, i, vp, vp, i64, vp, i64, vp, vp, vp, i64, i64, i64, i, vp, vp]
     _lib = lib

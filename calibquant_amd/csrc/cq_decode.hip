@@ -70,7 +70,11 @@ struct DecodeGeom {
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
 constexpr int cmin(int a, int b) { return a < b ? a : b; }
 
-template <int BITS, int HPB> struct Lay {
+// VTOK: values quantised per token and per group of 32 channels (scale * code + minimum,
+// codes in little-endian 32-bit words, first channel in the lowest bits) instead of per
+// channel.  A token slot then also carries the token's group scales, and every channel
+// group has its own subset-sum tables.
+template <int BITS, int HPB, bool VTOK = false> struct Lay {
     static constexpr int NB = 16 * BITS;            // bytes per packed row
     static constexpr int PC = NB * 8;               // bit lanes per row
     static constexpr int GPW = kWave / NB;          // 4-token groups per wave pass
@@ -80,7 +84,10 @@ template <int BITS, int HPB> struct Lay {
     static constexpr int HW = HPB >= 2 ? HPB / 2 : 1;   // 32-bit words per packed-fp16 entry
     static constexpr int ESZH = HW * 4;             // bytes per packed-fp16 table entry
     static constexpr int KT = NB * 256 * ESZ;       // K table bytes
-    static constexpr int WTAB = kNW * GPW * 16 * ESZH;
+    static constexpr int SLOT = VTOK ? 16 : ESZ;    // bytes per token slot: logits, later e (+ 4 group scales)
+    static constexpr int NGRP = VTOK ? kD / 32 : 1; // channel groups with tables of their own
+    static constexpr int WTAB = kNW * NGRP * GPW * 16 * ESZH;
+    static constexpr int RW = cmax(2 * HPB, VTOK ? NGRP * HPB : 0);   // widest block reduction
     static constexpr int VSUB = kNT * kPF / BITS;   // V tokens staged at a time
     static constexpr int KR = kPF / BITS;           // K token rounds in flight per thread
     static constexpr int RED = kNW * PC * ESZ;
@@ -91,8 +98,8 @@ template <int BITS, int HPB> struct Lay {
     static constexpr int F_QSZ = F_QF + HPB * kD;             // HPB*kD
     static constexpr int F_QRAW = F_QSZ + HPB * kD;           // HPB*kD raw 16-bit q
     static constexpr int F_RED = F_QRAW + HPB * kD / 2;       // kNW*HPB
-    static constexpr int F_STAT = F_RED + 2 * kNW * HPB;      // 8*HPB: per-head softmax state
-    static constexpr int F_VSZ = F_STAT + 8 * HPB;            // 2*kD: value scale, zero-point
+    static constexpr int F_STAT = F_RED + kNW * RW;           // 8*HPB: per-head softmax state
+    static constexpr int F_VSZ = F_STAT + 8 * HPB;            // 2*kD: value scale, zero-point (VTOK: NGRP*HPB minimum terms)
     static constexpr int F_NIB = F_VSZ + 2 * kD;              // NB*32*HPB: nibble tables
     static constexpr int F_SRES = F_NIB + NB * 32 * HPB;      // kResTile*HPB
     static constexpr int F_PRES = F_SRES + kResTile * HPB;    // kResTile*HPB
@@ -101,7 +108,7 @@ template <int BITS, int HPB> struct Lay {
     static constexpr int region_a(int cap) {
         return (cmax(cmax(KT, WTAB + cmin(VSUB, cap) * NB), cmax(RED, RED2)) + 255) / 256 * 256;
     }
-    static constexpr int lds_bytes(int cap) { return region_a(cap) + FIXED + cap * ESZ; }
+    static constexpr int lds_bytes(int cap) { return region_a(cap) + FIXED + cap * SLOT; }
     static constexpr int max_chunk() {
         int best = 64;
         for (int c = 64; c <= 16384; c += 64)
@@ -189,16 +196,17 @@ __device__ __forceinline__ uint32_t pack_f16(float a, float b) {
     return __builtin_bit_cast(uint32_t, h);
 }
 
-template <int BITS, int HPB, typename DT, bool MINMAX_ONLY>
+template <int BITS, int HPB, typename DT, bool MINMAX_ONLY, bool VTOK = false>
 __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
-    using L = Lay<BITS, HPB>;
+    using L = Lay<BITS, HPB, VTOK>;
     using V = Vec<HPB>;
     constexpr int NB = L::NB;
     extern __shared__ __attribute__((aligned(256))) unsigned char smem[];
     const int reg_a = L::region_a(g.cap);
     unsigned char* regA = smem;
     float* fx = reinterpret_cast<float*>(smem + reg_a);
-    V* logits = reinterpret_cast<V*>(smem + reg_a + L::FIXED);
+    unsigned char* slots = smem + reg_a + L::FIXED;   // one slot per token of the chunk
+    auto slot = [&](int t) { return slots + t * L::SLOT; };
     float* wbit = fx + L::F_WBIT;
     float* qf = fx + L::F_QF;
     float* qsz = fx + L::F_QSZ;
@@ -241,8 +249,8 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
         const uint16_t* qp = static_cast<const uint16_t*>(g.q) + (static_cast<int64_t>(b) * g.Hq + hq0) * kD;
         q_raw = qp[h * kD + d];
         const bool vstat = tid >= kNT - kD;   // the last kD threads fetch the value statistics
-        const uint16_t* sp = has_img ? static_cast<const uint16_t*>(vstat ? g.vs : g.ks) + bh * kD : qp;
-        const uint16_t* zp = has_img ? static_cast<const uint16_t*>(vstat ? g.vz : g.kz) + bh * kD : qp;
+        const uint16_t* sp = has_img ? static_cast<const uint16_t*>((vstat && !VTOK) ? g.vs : g.ks) + bh * kD : qp;
+        const uint16_t* zp = has_img ? static_cast<const uint16_t*>((vstat && !VTOK) ? g.vz : g.kz) + bh * kD : qp;
         s_raw = sp[d];
         z_raw = zp[d];
     }
@@ -309,7 +317,7 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
             }
         }
     }
-    if (n > 0 && tid >= kNT - kD && tid >= HPB * kD) {
+    if (!VTOK && n > 0 && tid >= kNT - kD && tid >= HPB * kD) {
         const int d = tid - (kNT - kD);
         fx[L::F_VSZ + d] = Cvt<DT>::to_float(s_raw);
         fx[L::F_VSZ + kD + d] = Cvt<DT>::to_float(z_raw);
@@ -543,7 +551,7 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                     if ((k & 7) == 7) __builtin_amdgcn_sched_barrier(0);
                 }
                 const V acc = part[5];
-                if constexpr (!MINMAX_ONLY) logits[tt] = acc;
+                if constexpr (!MINMAX_ONLY) *reinterpret_cast<V*>(slot(tt)) = acc;
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) { mn[h] = fminf(mn[h], acc.v[h]); mx[h] = fmaxf(mx[h], acc.v[h]); }
             }
@@ -665,14 +673,14 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) lm[h] = -INFINITY;
                 for (int tt = tid; tt < n; tt += kNT) {
-                    V w = logits[tt];
+                    V w = *reinterpret_cast<const V*>(slot(tt));
                     const float mv = mk[tt];
 #pragma unroll
                     for (int h = 0; h < HPB; ++h) {
                         w.v[h] = (w.v[h] - mn[h]) * slope[h] + tmin[h] + mv;
                         lm[h] = fmaxf(lm[h], w.v[h]);
                     }
-                    logits[tt] = w;
+                    *reinterpret_cast<V*>(slot(tt)) = w;
                 }
                 block_max<HPB>(lm, red);
 #pragma unroll
@@ -693,29 +701,54 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                 ec[h] = dead ? -INFINITY : (tmin[h] - m_img[h]) * kLog2e;
             }
             using HWv = Words<L::HW>;
+            // per-token value statistics (VTOK): (T, NGRP) scales and minima of this kv-head
+            const uint16_t* tsc = static_cast<const uint16_t*>(g.vs) + (bh * g.T + t0) * L::NGRP;
+            const uint16_t* tmn = static_cast<const uint16_t*>(g.vz) + (bh * g.T + t0) * L::NGRP;
+            float cma[VTOK ? L::NGRP * HPB : 1];   // sum_t e[t][h] * minimum[t][group], kept [group][head]
+#pragma unroll
+            for (int i = 0; i < (VTOK ? L::NGRP * HPB : 1); ++i) cma[i] = 0.f;
             for (int tt = tid; tt < npad; tt += kNT) {
                 float e[4] = {0.f, 0.f, 0.f, 0.f};
+                uint32_t sc2[2] = {0u, 0u};   // the token's group scales as fp16
                 if (tt < n) {
-                    const V w = logits[tt];
+                    const V w = *reinterpret_cast<const V*>(slot(tt));
 #pragma unroll
                     for (int h = 0; h < HPB; ++h) {
                         e[h] = __builtin_amdgcn_exp2f((w.v[h] - mn[h]) * ea[h] + ec[h]);
                         ls[h] += e[h];
+                    }
+                    if constexpr (VTOK) {
+                        const uint2 sr = *reinterpret_cast<const uint2*>(tsc + tt * L::NGRP);
+                        const uint2 mr = *reinterpret_cast<const uint2*>(tmn + tt * L::NGRP);
+                        sc2[0] = pack_f16(Cvt<DT>::lo(sr.x), Cvt<DT>::hi(sr.x));
+                        sc2[1] = pack_f16(Cvt<DT>::lo(sr.y), Cvt<DT>::hi(sr.y));
+                        const float mg[4] = {Cvt<DT>::lo(mr.x), Cvt<DT>::hi(mr.x), Cvt<DT>::lo(mr.y), Cvt<DT>::hi(mr.y)};
+#pragma unroll
+                        for (int gi = 0; gi < L::NGRP; ++gi)
+#pragma unroll
+                            for (int h = 0; h < HPB; ++h) cma[gi * HPB + h] += e[h] * mg[gi];
                     }
                 }
                 // e as packed fp16 in the first bytes of the token's slot (read by the V tables)
                 HWv hw;
                 hw.w[0] = pack_f16(e[0], e[1]);
                 if constexpr (L::HW == 2) hw.w[1] = pack_f16(e[2], e[3]);
-                *reinterpret_cast<HWv*>(&logits[tt]) = hw;
+                *reinterpret_cast<HWv*>(slot(tt)) = hw;
+                if constexpr (VTOK) *reinterpret_cast<uint2*>(slot(tt) + 8) = make_uint2(sc2[0], sc2[1]);
             }
             block_reduce<HPB>(ls, red, OpSum(), 0.f);   // its barriers also publish e and vst
+            if constexpr (VTOK) {
+                block_reduce<L::NGRP * HPB>(cma, red, OpSum(), 0.f);
+#pragma unroll
+                for (int i = 0; i < L::NGRP * HPB; ++i)
+                    if (tid == i) fx[L::F_VSZ + i] = cma[i];
+            }
 #pragma unroll
             for (int h = 0; h < HPB; ++h) l_img[h] = ls[h];
 
             // ---- phase 5: packed V ----------------------------------------------------------
             // lane = (byte column j, slice c of its 8 bit lanes); a wave pass covers TPW tokens
-            unsigned char* wtab = regA + wv * (L::GPW * 16 * L::ESZH);
+            unsigned char* wtab = regA + wv * (L::NGRP * L::GPW * 16 * L::ESZH);   // [channel group][token group][16]
             const int j = lane / L::GPW, cs = lane % L::GPW;
             const int bg = lane >> 4, be = lane & 15;   // table build: group, entry
             f16x2_t bsel[4];
@@ -746,6 +779,8 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                 bshr[m] = kInPlace ? 0u : sft;
             }
             using WG = Words<L::GPW>;   // the GPW dwords of one (unit, column)
+            // channel group of the lane's byte column (32 channels = 4*BITS columns): lane / 16 for both widths
+            const int cgrp = VTOK ? (lane >> 4) : 0;
             // absolute LDS address of the wave's tables (the dot product's addend)
             const uint32_t wtab_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
                 (__attribute__((address_space(3))) unsigned char*)wtab));
@@ -766,19 +801,38 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                     const int tl = u * L::TPW;        // token offset inside the block
                     if (bg < L::GPW) {
                         // entry `be` of group `bg`: fp16 sum of the e values its bits select
-                        f16x2_t val[L::HW];
+                        // (VTOK: of e times the token's scale for the channel group, per group)
+                        f16x2_t val[L::NGRP][L::HW];
 #pragma unroll
-                        for (int k = 0; k < L::HW; ++k) val[k] = f16x2_t{0, 0};
+                        for (int gi = 0; gi < L::NGRP; ++gi)
+#pragma unroll
+                            for (int k = 0; k < L::HW; ++k) val[gi][k] = f16x2_t{0, 0};
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
-                            const HWv e = *reinterpret_cast<const HWv*>(&logits[vs0 + tl + 4 * bg + i]);
+                            const unsigned char* sl = slot(vs0 + tl + 4 * bg + i);
+                            const HWv e = *reinterpret_cast<const HWv*>(sl);
+                            if constexpr (VTOK) {
+                                const uint2 sc = *reinterpret_cast<const uint2*>(sl + 8);
+                                const f16x2_t s01 = __builtin_bit_cast(f16x2_t, sc.x), s23 = __builtin_bit_cast(f16x2_t, sc.y);
+                                const _Float16 sg[4] = {s01.x, s01.y, s23.x, s23.y};
 #pragma unroll
-                            for (int k = 0; k < L::HW; ++k) val[k] += __builtin_bit_cast(f16x2_t, e.w[k]) * bsel[i];
+                                for (int gi = 0; gi < L::NGRP; ++gi) {
+                                    const f16x2_t w2 = bsel[i] * f16x2_t{sg[gi], sg[gi]};
+#pragma unroll
+                                    for (int k = 0; k < L::HW; ++k) val[gi][k] += __builtin_bit_cast(f16x2_t, e.w[k]) * w2;
+                                }
+                            } else {
+#pragma unroll
+                                for (int k = 0; k < L::HW; ++k) val[0][k] += __builtin_bit_cast(f16x2_t, e.w[k]) * bsel[i];
+                            }
                         }
-                        HWv o;
 #pragma unroll
-                        for (int k = 0; k < L::HW; ++k) o.w[k] = __builtin_bit_cast(uint32_t, val[k]);
-                        reinterpret_cast<HWv*>(wtab)[bg * 16 + be] = o;
+                        for (int gi = 0; gi < L::NGRP; ++gi) {
+                            HWv o;
+#pragma unroll
+                            for (int k = 0; k < L::HW; ++k) o.w[k] = __builtin_bit_cast(uint32_t, val[gi][k]);
+                            reinterpret_cast<HWv*>(wtab)[(gi * L::GPW + bg) * 16 + be] = o;
+                        }
                     }
                     const WG cw = *reinterpret_cast<const WG*>(vst + (u * NB + j) * L::TPW);
                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -790,7 +844,7 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                     f16x2_t pk[L::MPL][L::GPW][L::HW];
 #pragma unroll
                     for (int gq = 0; gq < L::GPW; ++gq) {
-                        const uint32_t tbase = wtab_addr + static_cast<uint32_t>(gq * 16 * L::ESZH);
+                        const uint32_t tbase = wtab_addr + static_cast<uint32_t>((cgrp * L::GPW + gq) * 16 * L::ESZH);
                         const uint32_t wsh = cw.w[gq] >> nib_shift;
 #pragma unroll
                         for (int m = 0; m < L::MPL; ++m) {
@@ -833,20 +887,29 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
             if (tid < HPB * kD) {
                 const int h = tid / kD, d = tid % kD;
                 float a = 0.f;
+                // bit lanes of channel d.  Per-channel codes: first channel of a byte in its top
+                // bits; per-token codes: first channel in the lowest bits.
+                const int per = 8 / BITS;                       // channels per byte
+                const int cb = d / per * 8, c = d % per;
+                const int lane_hi = VTOK ? cb + 8 - BITS * (c + 1) : cb + BITS * c;   // bit lane of the code's top bit
                 if constexpr (BITS == 1) {
 #pragma unroll
-                    for (int w = 0; w < kNW; ++w) a += redv[w * L::PC + d].v[h];
+                    for (int w = 0; w < kNW; ++w) a += redv[w * L::PC + lane_hi].v[h];
                 } else {
 #pragma unroll
                     for (int w = 0; w < kNW; ++w)
-                        a += 2.0f * redv[w * L::PC + 2 * d].v[h] + redv[w * L::PC + 2 * d + 1].v[h];
+                        a += 2.0f * redv[w * L::PC + lane_hi].v[h] + redv[w * L::PC + lane_hi + 1].v[h];
                 }
-                const float s = fx[L::F_VSZ + d];
-                const float z = fx[L::F_VSZ + kD + d];
-                float lh = l_img[0];
+                if constexpr (VTOK) {
+                    o_img = a + fx[L::F_VSZ + (d >> 5) * HPB + h];   // + sum_t e * minimum of the channel's group
+                } else {
+                    const float s = fx[L::F_VSZ + d];
+                    const float z = fx[L::F_VSZ + kD + d];
+                    float lh = l_img[0];
 #pragma unroll
-                for (int k = 1; k < HPB; ++k) lh = (h == k) ? l_img[k] : lh;
-                o_img = s * (a - z * lh);
+                    for (int k = 1; k < HPB; ++k) lh = (h == k) ? l_img[k] : lh;
+                    o_img = s * (a - z * lh);
+                }
             }
             __syncthreads();
         }
@@ -905,9 +968,9 @@ struct Plan {
     size_t ws_mm, ws_part;
 };
 
-template <int BITS, int HPB>
+template <int BITS, int HPB, bool VTOK>
 static void plan_for(const cq_decode_args* a, Plan* p) {
-    using L = Lay<BITS, HPB>;
+    using L = Lay<BITS, HPB, VTOK>;
     const int G = a->Hq / a->Hkv;
     const int64_t units = static_cast<int64_t>(a->B) * a->Hkv * (G / HPB);
     const int maxc = L::max_chunk();
@@ -947,25 +1010,27 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
     if (a->T < 0 || a->R < 0 || (a->T == 0 && a->R == 0)) return CQ_ERR_SHAPE;
     if (a->sprompt_len < 0 || a->sprompt_len > a->R) return CQ_ERR_SHAPE;
     const int G = a->Hq / a->Hkv;
+    if (a->v_mode != CQ_V_PER_CHANNEL && a->v_mode != CQ_V_PER_TOKEN) return CQ_ERR_UNSUPPORTED;
+    const bool vtok = a->v_mode == CQ_V_PER_TOKEN;
     if (a->bits == 1) {
-        if (G % 4 == 0) plan_for<1, 4>(a, p);
-        else if (G % 2 == 0) plan_for<1, 2>(a, p);
-        else plan_for<1, 1>(a, p);
+        if (G % 4 == 0) vtok ? plan_for<1, 4, true>(a, p) : plan_for<1, 4, false>(a, p);
+        else if (G % 2 == 0) vtok ? plan_for<1, 2, true>(a, p) : plan_for<1, 2, false>(a, p);
+        else vtok ? plan_for<1, 1, true>(a, p) : plan_for<1, 1, false>(a, p);
     } else {
-        if (G % 2 == 0) plan_for<2, 2>(a, p);
-        else plan_for<2, 1>(a, p);
+        if (G % 2 == 0) vtok ? plan_for<2, 2, true>(a, p) : plan_for<2, 2, false>(a, p);
+        else vtok ? plan_for<2, 1, true>(a, p) : plan_for<2, 1, false>(a, p);
     }
     const int64_t blocks = static_cast<int64_t>(a->B) * a->Hkv * (G / p->hpb) * p->nx;
     if (blocks > 0x7fffffff) return CQ_ERR_SHAPE;
     return CQ_OK;
 }
 
-template <int BITS, int HPB, typename DT>
+template <int BITS, int HPB, typename DT, bool VTOK>
 static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
     const int G = g.Hq / g.Hkv;
     const unsigned units = static_cast<unsigned>(g.B) * g.Hkv * (G / HPB);
-    auto kmain = decode_kernel<BITS, HPB, DT, false>;
-    auto kmm = decode_kernel<BITS, HPB, DT, true>;
+    auto kmain = decode_kernel<BITS, HPB, DT, false, VTOK>;
+    auto kmm = decode_kernel<BITS, HPB, DT, true, false>;   // the min/max pass never looks at values
     // raise the dynamic-LDS limit once per device for this instantiation
     static std::atomic<uint32_t> attr_done{0};
     int dev = 0;
@@ -982,7 +1047,7 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
         DecodeGeom g1 = g;
         g1.nx = g.nsplit;  // the min/max pass has no residual unit
         g1.cap = 0;        // ... and keeps no logits
-        const int lds_mm = Lay<BITS, HPB>::lds_bytes(0);
+        const int lds_mm = Lay<BITS, HPB, false>::lds_bytes(0);
         hipLaunchKernelGGL(kmm, dim3(units * g.nsplit), dim3(kNT), lds_mm, st, g1);
         CQ_LAUNCH_CHECK();
     }
@@ -996,15 +1061,15 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
     return CQ_OK;
 }
 
-template <typename DT>
+template <typename DT, bool VTOK>
 static int dispatch(const DecodeGeom& g, const Plan& p, int bits, hipStream_t st) {
     if (bits == 1) {
-        if (p.hpb == 4) return launch<1, 4, DT>(g, p, st);
-        if (p.hpb == 2) return launch<1, 2, DT>(g, p, st);
-        return launch<1, 1, DT>(g, p, st);
+        if (p.hpb == 4) return launch<1, 4, DT, VTOK>(g, p, st);
+        if (p.hpb == 2) return launch<1, 2, DT, VTOK>(g, p, st);
+        return launch<1, 1, DT, VTOK>(g, p, st);
     }
-    if (p.hpb == 2) return launch<2, 2, DT>(g, p, st);
-    return launch<2, 1, DT>(g, p, st);
+    if (p.hpb == 2) return launch<2, 2, DT, VTOK>(g, p, st);
+    return launch<2, 1, DT, VTOK>(g, p, st);
 }
 
 }  // namespace cq
@@ -1050,8 +1115,10 @@ int cq_decode_attn(const cq_decode_args* a, cq_stream_t stream) {
     g.cap = p.cap;
     g.one = 1.0f;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (a->dtype == CQ_BF16) return cq::dispatch<cq::BF16>(g, p, a->bits, st);
-    return cq::dispatch<cq::FP16>(g, p, a->bits, st);
+    const bool vtok = a->v_mode == CQ_V_PER_TOKEN;
+    if (a->dtype == CQ_BF16)
+        return vtok ? cq::dispatch<cq::BF16, true>(g, p, a->bits, st) : cq::dispatch<cq::BF16, false>(g, p, a->bits, st);
+    return vtok ? cq::dispatch<cq::FP16, true>(g, p, a->bits, st) : cq::dispatch<cq::FP16, false>(g, p, a->bits, st);
 }
 
 }  // extern "C"

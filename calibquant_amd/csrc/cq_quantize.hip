@@ -303,6 +303,66 @@ static int quant_entry(const void* x, int dtype, int B, int T, int H, int D, int
     return run_quant<FP16>(x, g, bits, clip, codes, xq, scale, zero, static_cast<float*>(ws), s);
 }
 
+// ---- per-token value quantiser --------------------------------------------------------
+// The reference's `triton_quantize_and_pack_along_last_dim` (qjl/new_pack.py:53-82): for every
+// token and every group of 32 consecutive channels min and max, scale = (max - min) / L,
+// code = round(clamp((x - min) / scale, 0, L)), every op rounded to the storage dtype
+// (`tensor / python int` multiplies by the fp32 reciprocal; `div_` by the scale tensor is an
+// IEEE division), 32/BITS codes per int32 word with the first code in the lowest bits.
+// 16 lanes cover a row of 128 channels with one 16-byte load each; the four lanes of a
+// quad are one group.  One pass over x.
+template <typename DT, int BITS>
+__global__ __launch_bounds__(kQThreads) void token_pack_kernel(const uint16_t* __restrict__ x, QuantGeom g,
+                                                               int32_t* __restrict__ words,
+                                                               uint16_t* __restrict__ scale,
+                                                               uint16_t* __restrict__ mins) {
+    constexpr float levels = static_cast<float>((1 << BITS) - 1);
+    const int64_t rows = static_cast<int64_t>(g.B) * g.H * g.T;
+    const int l16 = threadIdx.x & 15, q4 = threadIdx.x & 3, grp = l16 >> 2;
+    const float inv_levels = __fdiv_rn(1.0f, levels);
+    for (int64_t row = blockIdx.x * static_cast<int64_t>(kQThreads / 16) + (threadIdx.x >> 4); row < rows;
+         row += static_cast<int64_t>(gridDim.x) * (kQThreads / 16)) {
+        // output row order (b, h, t)
+        const int t = static_cast<int>(row % g.T);
+        const int h = static_cast<int>((row / g.T) % g.H);
+        const int b = static_cast<int>(row / (static_cast<int64_t>(g.T) * g.H));
+        const uint4 v = *reinterpret_cast<const uint4*>(x + b * g.sb + t * g.st + h * g.sh + l16 * 8);
+        float f[8];
+        unpack8<DT>(v, f);
+        float mn = f[0], mx = f[0];
+#pragma unroll
+        for (int i = 1; i < 8; ++i) { mn = fminf(mn, f[i]); mx = fmaxf(mx, f[i]); }
+        mn = quad_reduce(mn, OpMin(), INFINITY);
+        mx = quad_reduce(mx, OpMax(), -INFINITY);
+        const float s = rnd<DT>(rnd<DT>(mx - mn) * inv_levels);
+        uint32_t packed = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float y = rnd<DT>(f[i] - mn);
+            y = rnd<DT>(__fdiv_rn(y, s));
+            uint32_t code = 0;
+            if (y == y) code = static_cast<uint32_t>(rintf(fminf(fmaxf(y, 0.0f), levels)));
+            packed |= code << (BITS * i);
+        }
+        const int64_t gidx = row * (g.D / 32) + grp;
+        if constexpr (BITS == 1) {
+            // 8 bits per lane, 32 per quad: one word
+            uint32_t w = packed << (8 * q4);
+            w |= static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(w), 0xB1, 0xf, 0xf, true));   // lane ^ 1
+            w |= static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(w), 0x4E, 0xf, 0xf, true));   // lane ^ 2
+            if (q4 == 0) words[gidx] = static_cast<int32_t>(w);
+        } else {
+            // 16 bits per lane: lanes (0,1) and (2,3) of the quad make the group's two words
+            const uint32_t other = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(packed), 0xB1, 0xf, 0xf, true));
+            if ((q4 & 1) == 0) words[gidx * 2 + (q4 >> 1)] = static_cast<int32_t>(packed | (other << 16));
+        }
+        if (q4 == 0) {
+            scale[gidx] = static_cast<uint16_t>(Cvt<DT>::from_float(s));
+            mins[gidx] = static_cast<uint16_t>(Cvt<DT>::from_float(mn));
+        }
+    }
+}
+
 // ---- encode() ---------------------------------------------------------------------
 template <typename IT>
 __device__ __forceinline__ uint32_t index_of(const IT* p, int64_t i);
@@ -363,6 +423,40 @@ int cq_quantize_pack(const void* x, int dtype, int B, int T, int H, int D, int64
     if (!codes) return CQ_ERR_NULL;
     return cq::quant_entry(x, dtype, B, T, H, D, stride_b, stride_t, stride_h, bits, clip, codes, nullptr, scale,
                            zero, workspace, workspace_bytes, stream);
+}
+
+int cq_quantize_pack_token(const void* x, int dtype, int B, int T, int H, int D, int64_t stride_b, int64_t stride_t,
+                           int64_t stride_h, int bits, int group_size, int32_t* words, void* scale, void* mins,
+                           cq_stream_t stream) {
+    if (!x || !words || !scale || !mins) return CQ_ERR_NULL;
+    if (dtype != CQ_BF16 && dtype != CQ_FP16) return CQ_ERR_DTYPE;
+    if ((bits != 1 && bits != 2) || group_size != 32 || D != 128) return CQ_ERR_UNSUPPORTED;
+    if (B < 1 || T < 1 || H < 1) return CQ_ERR_SHAPE;
+    if ((stride_b % 8) || (stride_t % 8) || (stride_h % 8) || !cq::aligned16(x) ||
+        (reinterpret_cast<uintptr_t>(words) & 3u) || (reinterpret_cast<uintptr_t>(scale) & 1u) ||
+        (reinterpret_cast<uintptr_t>(mins) & 1u))
+        return CQ_ERR_ALIGN;
+    cq::QuantGeom g;
+    g.B = B; g.T = T; g.H = H; g.D = D;
+    g.sb = stride_b; g.st = stride_t; g.sh = stride_h;
+    g.nchunk = 1; g.chunk = T;
+    const int64_t rows = static_cast<int64_t>(B) * H * T;
+    int64_t blocks = (rows + cq::kQThreads / 16 - 1) / (cq::kQThreads / 16);
+    if (blocks > (1 << 20)) blocks = 1 << 20;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint16_t* xp = static_cast<const uint16_t*>(x);
+    uint16_t* sp = static_cast<uint16_t*>(scale);
+    uint16_t* mp = static_cast<uint16_t*>(mins);
+    const dim3 grid(static_cast<unsigned>(blocks)), block(cq::kQThreads);
+    if (dtype == CQ_BF16) {
+        if (bits == 1) hipLaunchKernelGGL((cq::token_pack_kernel<cq::BF16, 1>), grid, block, 0, st, xp, g, words, sp, mp);
+        else hipLaunchKernelGGL((cq::token_pack_kernel<cq::BF16, 2>), grid, block, 0, st, xp, g, words, sp, mp);
+    } else {
+        if (bits == 1) hipLaunchKernelGGL((cq::token_pack_kernel<cq::FP16, 1>), grid, block, 0, st, xp, g, words, sp, mp);
+        else hipLaunchKernelGGL((cq::token_pack_kernel<cq::FP16, 2>), grid, block, 0, st, xp, g, words, sp, mp);
+    }
+    CQ_LAUNCH_CHECK();
+    return CQ_OK;
 }
 
 int cq_quant(const void* x, int dtype, int B, int T, int H, int D, int64_t stride_b, int64_t stride_t,

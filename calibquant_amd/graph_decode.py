@@ -56,7 +56,8 @@ class _LayerState:
                                        att.encoded_features_v if T > 0 else None, stats[0], stats[1], stats[2],
                                        stats[3], self.kbuf, self.vbuf, sprompt_len=min(att.sprompt_len, R0),
                                        bits=att.bits_k, calibrate=att.normalize, calib_off_max=CALIB_OFFSET_MAX,
-                                       calib_off_min=CALIB_OFFSET_MIN, out=self.out, r_dev=r_len)
+                                       calib_off_min=CALIB_OFFSET_MIN, out=self.out, r_dev=r_len,
+                                       v_mode=getattr(att, "v_mode", "channel"))
 
 
 class StaticDecoder:

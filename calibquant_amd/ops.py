@@ -62,6 +62,27 @@ def quantize_pack(x: torch.Tensor, bits: int, clip: float) -> Tuple[torch.Tensor
     return codes, scale, zero
 
 
+def quantize_pack_token(x: torch.Tensor, bits: int, group_size: int = 32):
+    """Per-token min-max quantiser of the values (`v_mode = token`): x (B, T, H, D) view, bf16 or
+    fp16, D = 128, groups of 32 channels.  Returns words int32 (B, H, T, D*bits/32) (first channel
+    in the lowest bits), scale (B, H, T, D/32), mins (B, H, T, D/32); a value is scale*code + min."""
+    _need_gpu(x, "x")
+    dt = _storage_dtype(x, "x")
+    if x.dim() != 4 or x.stride(3) != 1:
+        raise _lib.CalibQuantError("x must be (B, T, H, D) with a contiguous last axis")
+    B, T, H, D = x.shape
+    lib = _lib.load()
+    words = torch.empty((B, H, T, D * bits // 32), dtype=torch.int32, device=x.device)
+    scale = torch.empty((B, H, T, D // group_size), dtype=x.dtype, device=x.device)
+    mins = torch.empty_like(scale)
+    with torch.cuda.device(x.device):
+        rc = lib.cq_quantize_pack_token(x.data_ptr(), dt, B, T, H, D, x.stride(0), x.stride(1), x.stride(2),
+                                        int(bits), int(group_size), words.data_ptr(), scale.data_ptr(),
+                                        mins.data_ptr(), _stream(x))
+    _lib.check(rc, "cq_quantize_pack_token")
+    return words, scale, mins
+
+
 def quant_codes(x: torch.Tensor, bits: int, clip: float):
     """The unfused quantiser: x (B, T, H, D) -> (x_q (B, T, H, D) of x.dtype
     holding the integer codes, scale (B, 1, H, D), zero (B, 1, H, D))."""
@@ -122,7 +143,7 @@ class DecodeCall:
 
     def __init__(self, q, codes_k, codes_v, k_scale, k_zero, v_scale, v_zero, k_res, v_res,
                  sprompt_len=0, bits=1, calibrate=True, calib_off_max=-3.0, calib_off_min=0.0,
-                 mask=None, out=None, force_splits=0, r_dev=None):
+                 mask=None, out=None, force_splits=0, r_dev=None, v_mode="channel"):
         _need_gpu(q, "q")
         dt = _storage_dtype(q, "q")
         if q.dim() != 3:
@@ -143,6 +164,12 @@ class DecodeCall:
                 if t.dtype != q.dtype:
                     raise _lib.CalibQuantError("scale / zero-point dtype must match q")
             Hkv, T = codes_k.shape[1], codes_k.shape[2]
+            if v_mode == "token":
+                # values in the per-token layout of quantize_pack_token: int32 words, (T, D/32) scale and minimum
+                if codes_v.dtype != torch.int32 or codes_v.shape != (B, Hkv, T, D * int(bits) // 32):
+                    raise _lib.CalibQuantError("v_mode='token': codes_v must be int32 (B, Hkv, T, D*bits/32)")
+                if v_scale.shape != (B, Hkv, T, D // 32) or v_zero.shape != v_scale.shape:
+                    raise _lib.CalibQuantError("v_mode='token': v_scale / v_zero must be (B, Hkv, T, D/32)")
             a.codes_k, a.codes_v = codes_k.data_ptr(), codes_v.data_ptr()
             a.k_scale, a.k_zero = k_scale.data_ptr(), k_zero.data_ptr()
             a.v_scale, a.v_zero = v_scale.data_ptr(), v_zero.data_ptr()
@@ -177,6 +204,9 @@ class DecodeCall:
         a.calibrate = int(bool(calibrate))
         a.calib_off_max, a.calib_off_min = float(calib_off_max), float(calib_off_min)
         a.force_splits = int(force_splits)
+        if v_mode not in ("channel", "token"):
+            raise _lib.CalibQuantError("v_mode must be 'channel' or 'token'")
+        a.v_mode = 1 if v_mode == "token" else 0
         if r_dev is not None:
             # residual row count read on the device at run time; k_res / v_res are then the
             # whole window buffers (capacity rows) and R is that capacity
@@ -221,16 +251,18 @@ def decode_attn(q: torch.Tensor, codes_k: Optional[torch.Tensor], codes_v: Optio
                 sprompt_len: int = 0, bits: int = 1, calibrate: bool = True,
                 calib_off_max: float = -3.0, calib_off_min: float = 0.0,
                 mask: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
-                force_splits: int = 0, r_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
+                force_splits: int = 0, r_dev: Optional[torch.Tensor] = None,
+                v_mode: str = "channel") -> torch.Tensor:
     """One decode-attention step over packed image K/V plus the fp residual window.
 
     q (B, Hq, D); codes_* uint8 (B, Hkv, T, D*bits/8); *_scale, *_zero (B, Hkv, D);
     k_res, v_res (B, Hkv, R, D) (any b/h/r strides); mask optional additive
     (B, S + T + R - S) over the [sys | image | text] order.  `r_dev` (int32 GPU scalar): the
     number of valid rows of k_res / v_res, read on the device when the launch runs.
+    `v_mode='token'`: codes_v / v_scale / v_zero as returned by `quantize_pack_token`.
     Returns (B, Hq, D)."""
     call = DecodeCall(q, codes_k, codes_v, k_scale, k_zero, v_scale, v_zero, k_res, v_res,
-                      sprompt_len, bits, calibrate, calib_off_max, calib_off_min, mask, out, force_splits, r_dev)
+                      sprompt_len, bits, calibrate, calib_off_max, calib_off_min, mask, out, force_splits, r_dev, v_mode)
     with torch.cuda.device(call.device):
         return call.run()
 

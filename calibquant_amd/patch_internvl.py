@@ -122,7 +122,11 @@ def forward_internlm2_calibquant(self, hidden_states: torch.Tensor, attention_ma
     one_bit = self.bits_k == 1
     self.scale_k = getattr(self, "cq_scale_k", 0.5 if one_bit else 1)
     self.scale_v = getattr(self, "cq_scale_v", 0.3 if one_bit else 1)
-    self.per_channel_k = self.per_channel_v = True
+    # values: per channel (CalibQuant) or per token in groups of 32 channels (the layout of
+    # qjl/new_pack.py:53-82 that the reference's per-token branch reads, patch_internvl.py:560-577)
+    self.v_mode = getattr(self, "cq_v_mode", "channel")
+    self.per_channel_k = True
+    self.per_channel_v = self.v_mode == "channel"
     self.image_token_num = _image_token_num(self)
     self.normalize = self.bits_k <= 2
     if "padding_mask" in kwargs:
@@ -161,14 +165,20 @@ def forward_internlm2_calibquant(self, hidden_states: torch.Tensor, attention_ma
             k_img = key_states[:, :, S:S + T, :].transpose(1, 2)      # (B, T, Hkv, D) strided views
             v_img = value_states[:, :, S:S + T, :].transpose(1, 2)
             ck, ks, kz = ops.quantize_pack(k_img, self.bits_k, self.scale_k)
-            cv, vs, vz = ops.quantize_pack(v_img, self.bits_v, self.scale_v)
+            if self.v_mode == "token":
+                cv, vs, vz = ops.quantize_pack_token(v_img, self.bits_v)      # words, scale, minimum per (token, group)
+            else:
+                cv, vs, vz = ops.quantize_pack(v_img, self.bits_v, self.scale_v)
             self.encoded_features_k, self.encoded_features_v = ck, cv
             self._cq_stats = (ks, kz, vs, vz)                          # compact (B, Hkv, D)
             # reference-shaped views of the statistics: (B, Hq, 1, D) after repeat_kv (patch_internvl.py:300-309)
             self.scale_key = repeat_kv(ks.unsqueeze(2), G)
             self.zero_point_key = repeat_kv(kz.unsqueeze(2), G)
-            self.scale_value = repeat_kv(vs.unsqueeze(2), G)
-            self.zero_point_value = repeat_kv(vz.unsqueeze(2), G)
+            if self.v_mode == "token":
+                self.scale_value, self.zero_point_value = repeat_kv(vs, G), repeat_kv(vz, G)   # (B, Hq, T, D/32)
+            else:
+                self.scale_value = repeat_kv(vs.unsqueeze(2), G)
+                self.zero_point_value = repeat_kv(vz.unsqueeze(2), G)
             lut = torch.arange(2 ** self.bits_k, device=hidden_states.device, dtype=hidden_states.dtype)
             self.unique_values_k, self.unique_values_v = lut, lut.half()
         else:
@@ -216,7 +226,8 @@ def forward_internlm2_calibquant(self, hidden_states: torch.Tensor, attention_ma
         call = ops.DecodeCall(q1, self.encoded_features_k if T > 0 else None,
                               self.encoded_features_v if T > 0 else None, stats[0], stats[1], stats[2], stats[3],
                               k_res, v_res, sprompt_len=min(S, R), bits=self.bits_k, calibrate=self.normalize,
-                              calib_off_max=CALIB_OFFSET_MAX, calib_off_min=CALIB_OFFSET_MIN, mask=mask)
+                              calib_off_max=CALIB_OFFSET_MAX, calib_off_min=CALIB_OFFSET_MIN, mask=mask,
+                              v_mode=self.v_mode)
         with torch.cuda.device(call.device):
             out = call.run()
         self._cq_call = call if mask is None else None
@@ -238,7 +249,7 @@ def patch_model(model, quant_method="calibquant", **kwargs):
     """Route a chat model's generate and its attention forward to the quantised-KV path
     (patch_internvl.py:645-660).  Works on any object exposing
     `language_model.model.layers[i].attention` and a class-level `generate`.
-    Optional keyword overrides: bits, scale_k, scale_v, sprompt_len."""
+    Optional keyword overrides: bits, scale_k, scale_v, sprompt_len, v_mode ("channel" | "token")."""
     if quant_method not in ATTN_FORWARD_FUNCTIONS:
         raise KeyError(quant_method)
     if quant_method == "qjl":
@@ -248,7 +259,7 @@ def patch_model(model, quant_method="calibquant", **kwargs):
     print(f"Patching InternLM2FlashAttention2.forward function ... {quant_method}")
     layers = model.language_model.model.layers
     layers[0].attention.__class__.forward = ATTN_FORWARD_FUNCTIONS[quant_method]
-    for name in ("bits", "scale_k", "scale_v", "sprompt_len"):
+    for name in ("bits", "scale_k", "scale_v", "sprompt_len", "v_mode"):
         if name in kwargs:
             for layer in layers:
                 setattr(layer.attention, "cq_" + name, kwargs[name])

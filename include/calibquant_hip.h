@@ -66,6 +66,22 @@ int cq_quantize_pack(const void* x, int dtype, int B, int T, int H, int D,
                      uint8_t* codes, void* scale, void* zero,
                      void* workspace, size_t workspace_bytes, cq_stream_t stream);
 
+/* ------------------------------------------------------------------------
+ * Per-token value quantiser: the reference's
+ * triton_quantize_and_pack_along_last_dim(data, group_size, bit)
+ * (qjl/new_pack.py:53-82), the source of the `v_mode = token` layout that
+ * cq_decode_attn reads with CQ_V_PER_TOKEN.  x: (B, T, H, D) through element
+ * strides (D contiguous, D = 128, group_size = 32); for every token and group
+ * of 32 channels: minimum, scale = (max - min) / (2^bits - 1), code =
+ * round(clamp((x - min) / scale, 0, 2^bits - 1)), each op rounded to the
+ * storage dtype; 32/bits codes per int32 word, first code in the lowest bits
+ * (new_pack.py:7-28).  Outputs in (b, h, t) row order: words
+ * (B, H, T, D*bits/32), scale and mins (B, H, T, D/32) in the storage dtype.
+ * A value is scale*code + min (quantization.cu:116-117). */
+int cq_quantize_pack_token(const void* x, int dtype, int B, int T, int H, int D, int64_t stride_b,
+                           int64_t stride_t, int64_t stride_h, int bits, int group_size, int32_t* words,
+                           void* scale, void* mins, cq_stream_t stream);
+
 /* quant() itself, for callers that keep the reference's unfused call sequence
  * (calibquant.py:24-42 with per_channel=True, post_scale=True).  x_q is a
  * contiguous (B, T, H, D) tensor of storage dtype holding the integer codes
@@ -97,6 +113,9 @@ int cq_lut_vecmat_qk(const void* lut, int lut_dtype, const void* a, int a_dtype,
 int cq_lut_vecmat_pv(const void* lut, int lut_dtype, const void* a, int a_dtype,
                      const uint8_t* enc, int64_t M, int T, int D, int bits,
                      void* out_fp16, cq_stream_t stream);
+
+/* value quantisation layouts understood by cq_decode_attn (cq_decode_args.v_mode) */
+enum cq_v_mode { CQ_V_PER_CHANNEL = 0, CQ_V_PER_TOKEN = 1 };
 
 /* ------------------------------------------------------------------------
  * Decode: one fused attention step over packed image K/V plus the
@@ -152,6 +171,14 @@ typedef struct cq_decode_args {
      * every step (patch_internvl.py:246-251,265-266), which a recorded
      * launch cannot.  Must be NULL when a mask is given. */
     const int32_t* r_dev;
+    /* How the values were quantised (enum cq_v_mode).  CQ_V_PER_CHANNEL (0):
+     * CalibQuant's per-channel statistics, fields as described above.
+     * CQ_V_PER_TOKEN: the per-token layout of cq_quantize_pack_token (the
+     * reference's qjl/new_pack.py:53-82, consumed by quantization.cu:67-132):
+     * codes_v then holds int32 words (B, Hkv, T, D*bits/32), first channel in
+     * the lowest bits; v_scale and v_zero hold the scale and the minimum,
+     * storage dtype, (B, Hkv, T, D/32); a value is scale*code + minimum. */
+    int v_mode;
 } cq_decode_args;
 
 size_t cq_decode_attn_workspace(const cq_decode_args* args);

@@ -240,7 +240,7 @@ def decode_attention(q, codes_k, codes_v, k_scale, k_zero, v_scale, v_zero,
                      k_res, v_res, sprompt_len: int, bits: int,
                      off_max: float = -3.0, off_min: float = 0.0,
                      calibrate_logits: bool = True, mask=None,
-                     ftype=np.float32) -> np.ndarray:
+                     ftype=np.float32, v_token_group: int = 0) -> np.ndarray:
     """Dequant-attention oracle for one decode step, computed in `ftype` from
     the packed codes and the stored scales / zero-points.
 
@@ -255,7 +255,12 @@ def decode_attention(q, codes_k, codes_v, k_scale, k_zero, v_scale, v_zero,
     calibration of the image logits only (:376-385); concatenation
     [sys | image | text] (:388); additive mask (:404-410); softmax (:413);
     image output s_v (sum p code) - s_v z_v sum p (:418-425); residual
-    outputs (:428-434); sum (:434).  Returns (B, Hq, D) in `ftype`."""
+    outputs (:428-434); sum (:434).  Returns (B, Hq, D) in `ftype`.
+
+    `v_token_group` > 0: the values are in the per-token layout of
+    `kivi_quantize_pack` instead (codes_v int32 words, v_scale / v_zero the
+    (B, Hkv, T, D/group) scale and minimum) and dequantise as
+    scale*code + minimum (quantization.cu:116-117)."""
     q = np.asarray(q, dtype=ftype)
     B, Hq, D = q.shape
     Hkv = codes_k.shape[1]
@@ -268,9 +273,14 @@ def decode_attention(q, codes_k, codes_v, k_scale, k_zero, v_scale, v_zero,
     with np.errstate(all="ignore"):
         if T:
             ck = unpack(codes_k, bits).astype(ftype)
-            cv = unpack(codes_v, bits).astype(ftype)
             khat = np.asarray(k_scale, ftype)[:, :, None, :] * (ck - np.asarray(k_zero, ftype)[:, :, None, :])
-            vhat = np.asarray(v_scale, ftype)[:, :, None, :] * (cv - np.asarray(v_zero, ftype)[:, :, None, :])
+            if v_token_group:
+                cv = kivi_unpack(codes_v, bits).astype(ftype)
+                vhat = (np.repeat(np.asarray(v_scale, ftype), v_token_group, axis=-1) * cv
+                        + np.repeat(np.asarray(v_zero, ftype), v_token_group, axis=-1))
+            else:
+                cv = unpack(codes_v, bits).astype(ftype)
+                vhat = np.asarray(v_scale, ftype)[:, :, None, :] * (cv - np.asarray(v_zero, ftype)[:, :, None, :])
             w_img = np.einsum("bhd,bhtd->bht", q, repeat_kv(khat, G)) * inv
             if calibrate_logits:
                 w_img = calibrate(w_img, off_max, off_min, ftype)

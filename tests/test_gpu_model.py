@@ -185,3 +185,37 @@ def test_static_decoder_graph_replays_equal_eager_steps(quantized):
             assert ((w.max(-1).values - w.gather(1, got_tok[:, None])[:, 0]) < 0.15).all()
     finally:
         InternLM2Attention.forward, InternVLChatStandIn.generate = fp_forward, fp_generate
+
+
+def test_patched_model_with_per_token_values():
+    """`patch_model(..., v_mode="token")`: values quantised per token at prefill, decoded by the
+    fused kernel; one layer's decode output against the oracle on the module's own state."""
+    from calibquant_amd import patch_internvl as pi
+    from calibquant_amd.internlm2 import InternLM2Attention, InternLM2Config
+    torch.manual_seed(9)
+    cfg = InternLM2Config.tiny()
+    att = InternLM2Attention(cfg).cuda().to(torch.bfloat16)
+    att.cq_sprompt_len, att.image_token_num, att.cq_v_mode = 4, 300, "token"
+    B, S, T, TXT = 2, 4, 300, 6
+    N = S + T + TXT
+    x = torch.randn(B, N, cfg.hidden_size, device="cuda", dtype=torch.bfloat16)
+    pos = torch.arange(N, device="cuda")[None].expand(B, N)
+    with torch.no_grad():
+        _, _, past = pi.forward_internlm2_calibquant(att, x, None, pos, None, False, True)
+        assert att.encoded_features_v.dtype == torch.int32 and att.encoded_features_v.shape == (B, 2, T, 4)
+        assert att.scale_value.shape == (B, cfg.num_attention_heads, T, 4)
+        _, _, v = att.split_qkv(x)
+        w_ref, s_ref, m_ref = O.kivi_quantize_pack(to_np(v[:, S:S + T].transpose(1, 2)), 32, 1, "bf16")
+        assert np.array_equal(att.encoded_features_v.cpu().numpy(), w_ref)
+        xd = torch.randn(B, 1, cfg.hidden_size, device="cuda", dtype=torch.bfloat16)
+        posd = torch.full((B, 1), N, device="cuda", dtype=torch.long)
+        out_d, _, past2 = pi.forward_internlm2_calibquant(att, xd, None, posd, past, False, True)
+        qd, kd, vd = att.split_qkv(xd)
+        cos, sin = att.rotary_emb(vd, seq_len=N + 1)
+        qd, kd = pi.apply_rotary_pos_emb(qd.transpose(1, 2), kd.transpose(1, 2), cos, sin, posd)
+        ks, kz, _, _ = att._cq_stats
+        want = O.decode_attention(to_np(qd[:, :, 0]), att.encoded_features_k.cpu().numpy(), w_ref, to_np(ks), to_np(kz),
+                                  s_ref, m_ref, to_np(past2[0]), to_np(past2[1]), S, 1, v_token_group=32)
+        ref = att.wo(torch.from_numpy(want).cuda().to(torch.bfloat16).reshape(B, 1, -1))
+        err = (out_d.float() - ref.float()).abs()
+        assert err.max().item() < 2e-2 and err.mean().item() < 2e-3

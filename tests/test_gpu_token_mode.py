@@ -1,0 +1,83 @@
+"""Per-token value layout (`v_mode = token`, the reference's qjl/new_pack.py:53-82 quantiser and
+its consumer quantization.cu:67-132): bit-exact words / scales / minima against the oracle, and the
+fused decode kernel reading that layout against the fp32 dequant-attention oracle
+(1e-2 max-abs, 1e-3 mean-abs)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import cq_oracle as O
+from tests.util import case_to_gpu, make_case, same_bits, to_gpu, to_np
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, MEAN_ABS = 1e-2, 1e-3
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("bits", [1, 2])
+def test_quantize_pack_token_is_bit_exact(bits, dtype):
+    from calibquant_amd import ops
+    B, T, H, D = 2, 333, 3, 128
+    k, v = O.synth_kv(B, T, H, D, dtype, seed=31)
+    v[0, 5, 1, 32:64] = v[0, 5, 1, 32]            # a constant group: scale 0, codes from NaN -> 0
+    # a strided view, as the value block of a fused projection output is
+    wide = torch.zeros((B, T, H, 3, D), dtype=to_gpu(v, dtype).dtype, device="cuda")
+    wide[:, :, :, 2] = to_gpu(v, dtype)
+    words, scale, mins = ops.quantize_pack_token(wide[:, :, :, 2], bits)
+    torch.cuda.synchronize()
+    w_ref, s_ref, m_ref = O.kivi_quantize_pack(np.transpose(v, (0, 2, 1, 3)), 32, bits, dtype)
+    assert words.shape == (B, H, T, D * bits // 32) and words.dtype == torch.int32
+    assert np.array_equal(words.cpu().numpy(), w_ref)
+    assert same_bits(to_np(scale), s_ref) and same_bits(to_np(mins), m_ref)
+
+
+def _token_case(B, Hq, Hkv, T, R, bits, dtype, seed):
+    c = make_case(B, Hq, Hkv, 128, T, R, bits, dtype, seed)
+    words, scale, mins = O.kivi_quantize_pack(np.transpose(c["v"], (0, 2, 1, 3)), 32, bits, dtype)
+    c["cv"], c["sv"], c["zv"] = words, scale, mins
+    return c
+
+
+CASES = [
+    # B, Hq, Hkv, T, R, S
+    (2, 32, 8, 3328, 128, 0),      # InternVL2.5-8B layer shape, small batch (one chunk of tokens)
+    (2, 32, 8, 777, 60, 41),       # ragged T, system prompt rows
+    (1, 48, 8, 1000, 33, 0),       # six q heads per kv head
+    (1, 8, 8, 130, 0, 0),          # one q head per kv head, no residual
+]
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("bits", [1, 2])
+@pytest.mark.parametrize("case", CASES)
+def test_decode_attn_token_values_match_oracle(case, bits, dtype):
+    from calibquant_amd import ops
+    B, Hq, Hkv, T, R, S = case
+    c = _token_case(B, Hq, Hkv, T, R, bits, dtype, seed=40 + T)
+    g = case_to_gpu(c, dtype)
+    out = ops.decode_attn(g["q"], g["ck"], g["cv"], g["sk"], g["zk"], g["sv"], g["zv"],
+                          g["kr"] if R else None, g["vr"] if R else None, sprompt_len=S, bits=bits, v_mode="token")
+    torch.cuda.synchronize()
+    want = O.decode_attention(c["q"], c["ck"], c["cv"], c["sk"], c["zk"], c["sv"], c["zv"],
+                              c["kr"] if R else None, c["vr"] if R else None, S, bits, v_token_group=32)
+    err = np.abs(to_np(out) - want)
+    assert np.isfinite(to_np(out)).all()
+    assert err.max() < MAX_ABS and err.mean() < MEAN_ABS, (err.max(), err.mean())
+
+
+@pytest.mark.parametrize("bits", [1, 2])
+def test_decode_attn_token_values_split_path(bits):
+    """The chunked path (min/max launch, partials, merge) with per-token values."""
+    from calibquant_amd import ops
+    B, Hq, Hkv, T, R, S = 1, 32, 8, 5000, 70, 3
+    c = _token_case(B, Hq, Hkv, T, R, bits, "bf16", seed=77)
+    g = case_to_gpu(c, "bf16")
+    want = O.decode_attention(c["q"], c["ck"], c["cv"], c["sk"], c["zk"], c["sv"], c["zv"], c["kr"], c["vr"], S, bits,
+                              v_token_group=32)
+    for splits in (0, 3):
+        out = ops.decode_attn(g["q"], g["ck"], g["cv"], g["sk"], g["zk"], g["sv"], g["zv"], g["kr"], g["vr"],
+                              sprompt_len=S, bits=bits, v_mode="token", force_splits=splits)
+        torch.cuda.synchronize()
+        err = np.abs(to_np(out) - want)
+        assert err.max() < MAX_ABS and err.mean() < MEAN_ABS, (splits, err.max(), err.mean())

@@ -45,7 +45,12 @@ def test_c_abi_rejects_bad_arguments_without_touching_the_gpu():
     a.T, a.B = 32768, 8
     ws = lib.cq_decode_attn_workspace(ctypes.byref(a))
     assert ws > 0 and ws % 4 == 0                                         # chunked path needs partials
-    assert lib.cq_quantize_pack_workspace(64, 3328, 8, 128) == 64 * 8 * 8 * 2 * 128 * 4
+    # 8 token chunks of partial min / max, then 3 thresholds per channel
+    assert lib.cq_quantize_pack_workspace(64, 3328, 8, 128) == 64 * 8 * (8 * 2 + 3) * 128 * 4
+    a.T, a.B, a.v_mode = 64, 1, 7
+    assert lib.cq_decode_attn(ctypes.byref(a), None) == -7                # unknown value layout
+    assert lib.cq_quantize_pack_token(None, 0, 1, 1, 1, 128, 0, 0, 0, 1, 32, None, None, None, None) == -1
+    assert lib.cq_rope_append(None, 0, 1, 32, 8, 128, None, None, 1, None, 1, None, None, None, 0, 0, 0, 1, None, None) == -1
     assert lib.cq_quantize_pack(None, 0, 1, 1, 1, 128, 0, 0, 0, 1, 0.5, None, None, None, None, 0, None) == -1
     assert lib.cq_encode(None, 3, 1, 128, 1, None, None) == -1
 
