@@ -127,6 +127,49 @@ def time_fp16_kv(torch, shape, steps, warmup, nsets):
     return start.elapsed_time(end) / steps
 
 
+def _time_fn(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / steps
+
+
+def side_legs(torch, ops, shape, bits, sets):
+    """Figures next to the headline one, same layer shape: the prefill quantise-and-pack of one
+    K tensor read as the strided key block of a fused projection output (read-once roofline),
+    and the decode kernel on per-token values (`v_mode = token`)."""
+    B, Hq, Hkv, D, T, R, S = shape
+    dev = torch.device("cuda:0")
+    G = Hq // Hkv
+    res = {}
+    proj = torch.randn((B, T, Hkv, G + 2, D), device=dev, dtype=torch.bfloat16)
+    k_view, v_view = proj[..., -2, :], proj[..., -1, :]
+    clip = 0.5 if bits == 1 else 1.0
+    ms = _time_fn(torch, lambda: ops.quantize_pack(k_view, bits, clip), 10, 3)
+    rd = B * T * Hkv * D * 2 + B * Hkv * T * D * bits // 8
+    res["prefill_quantize_pack"] = {"us_per_tensor": round(ms * 1e3, 1), "algorithmic_bytes": rd,
+                                    "achieved_GBps": round(rd / ms / 1e6, 1),
+                                    "frac_of_hbm_peak": round(rd / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    ms_t = _time_fn(torch, lambda: ops.quantize_pack_token(v_view, bits), 10, 3)
+    words, vsc, vmn = ops.quantize_pack_token(v_view, bits)
+    del proj, k_view, v_view
+    s0 = sets[0]
+    call = ops.DecodeCall(s0["q"], s0["ck"], words, s0["sk"], s0["zk"], vsc, vmn, s0["kr"], s0["vr"],
+                          sprompt_len=S, bits=bits, v_mode="token")
+    ms_d = _time_fn(torch, call.run, 100, 10)
+    nb = algorithmic_bytes(B, Hq, Hkv, D, T, R, bits) - 2 * B * Hkv * D * 2 + 2 * B * Hkv * T * (D // 32) * 2
+    res["per_token_values"] = {"quantize_pack_token_us": round(ms_t * 1e3, 1), "decode_us_layer": round(ms_d * 1e3, 2),
+                               "algorithmic_bytes": nb, "achieved_GBps": round(nb / ms_d / 1e6, 1),
+                               "note": "one buffer set (codes may be served from the Infinity Cache)"}
+    return res
+
+
 def cpu_baseline(torch, sets, shape, bits, budget_s=12.0):
     """C port of the oracle on this host's cores, on a bounded sample: the
     first `bs` batch rows of the workload; the per-layer figure is scaled
@@ -284,6 +327,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-fp16kv", action="store_true", help="skip the fp16-KV comparison leg")
     ap.add_argument("--no-model", action="store_true", help="skip the full-model decode tok/s leg")
+    ap.add_argument("--no-side", action="store_true", help="skip the prefill / per-token-value side figures")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch three 256 MiB device copies (known traffic, for scaling profiler byte counters)")
     ap.add_argument("--seed", type=int, default=1234)
@@ -344,6 +388,11 @@ def main():
             out["fp16_kv_error"] = repr(e)[:200]
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline(torch, sets, shape, a.bits)
+    if not a.no_side:
+        try:
+            out["side_legs"] = side_legs(torch, ops, shape, a.bits, sets)
+        except Exception as e:  # side figures must not sink the measurement
+            out["side_legs"] = {"error": repr(e)[:300]}
     if not a.no_model and a.workload == DEFAULT_WORKLOAD and a.bits == 1:
         del sets, calls
         torch.cuda.empty_cache()
