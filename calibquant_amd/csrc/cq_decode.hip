@@ -87,7 +87,7 @@ template <int BITS, int HPB, bool VTOK = false> struct Lay {
     static constexpr int SLOT = VTOK ? 16 : ESZ;    // bytes per token slot: logits, later e (+ 4 group scales)
     static constexpr int NGRP = VTOK ? kD / 32 : 1; // channel groups with tables of their own
     static constexpr int WTAB = kNW * NGRP * GPW * 16 * ESZH;
-    static constexpr int RW = cmax(2 * HPB, VTOK ? NGRP * HPB : 0);   // widest block reduction
+    static constexpr int RW = cmax(2 * HPB, VTOK ? (NGRP + 1) * HPB : 0);   // widest set of per-wave partials
     static constexpr int VSUB = kNT * kPF / BITS;   // V tokens staged at a time
     static constexpr int KR = kPF / BITS;           // K token rounds in flight per thread
     static constexpr int RED = kNW * PC * ESZ;
@@ -437,7 +437,15 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
     float mn[HPB], mx[HPB];
 #pragma unroll
     for (int h = 0; h < HPB; ++h) { mn[h] = INFINITY; mx[h] = -INFINITY; }
-    U4 vc[kPF];   // first block of packed V rows, requested as the packed K registers free up
+    // First block of packed V rows: half of it is requested here, behind the packed K rows, the
+    // rest as the K registers free up, so it has arrived when the logits are done.
+    U4 vc[kPF];
+    auto request_v = [&](int r) { vc[r] = cvp4[min((tid + (r / BITS) * kNT) * BITS + r % BITS, last_u)]; };
+    constexpr int kVEarly = kPF / 2;
+    if constexpr (!MINMAX_ONLY) {
+#pragma unroll
+        for (int r = 0; r < kVEarly; ++r) request_v(r);
+    }
 
     if (n > 0) {
         // ---- phase 2: byte table = high-nibble table + low-nibble table ----------------
@@ -563,9 +571,8 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
         if constexpr (L::KR > (R)) {                                                          \
             token_logits(tid + (R) * kNT, kc[(R)]);                                           \
             if constexpr (!MINMAX_ONLY) {                                                     \
-                vc[(R) * BITS] = cvp4[min((tid + (R) * kNT) * BITS, last_u)];                 \
-                if constexpr (BITS == 2)                                                      \
-                    vc[(R) * BITS + 1] = cvp4[min((tid + (R) * kNT) * BITS + 1, last_u)];     \
+                if constexpr (kVEarly + (R) * BITS < kPF) request_v(kVEarly + (R) * BITS);        \
+                if constexpr (BITS == 2 && kVEarly + (R) * BITS + 1 < kPF) request_v(kVEarly + (R) * BITS + 1); \
             }                                                                                 \
         }
         CQ_K_ROUND(0)
@@ -605,9 +612,9 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
         }
         return;
     } else {
-        float m_img[HPB], l_img[HPB];
+        float m_img[HPB];
 #pragma unroll
-        for (int h = 0; h < HPB; ++h) { m_img[h] = -INFINITY; l_img[h] = 0.f; }
+        for (int h = 0; h < HPB; ++h) m_img[h] = -INFINITY;
         float o_img = 0.f;  // thread (h, d) = (tid / kD, tid % kD) for tid < HPB*kD
 
         if (n > 0) {
@@ -736,15 +743,10 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                 *reinterpret_cast<HWv*>(slot(tt)) = hw;
                 if constexpr (VTOK) *reinterpret_cast<uint2*>(slot(tt) + 8) = make_uint2(sc2[0], sc2[1]);
             }
-            block_reduce<HPB>(ls, red, OpSum(), 0.f);   // its barriers also publish e and vst
-            if constexpr (VTOK) {
-                block_reduce<L::NGRP * HPB>(cma, red, OpSum(), 0.f);
-#pragma unroll
-                for (int i = 0; i < L::NGRP * HPB; ++i)
-                    if (tid == i) fx[L::F_VSZ + i] = cma[i];
-            }
-#pragma unroll
-            for (int h = 0; h < HPB; ++h) l_img[h] = ls[h];
+            // The sums of e (and of e * minimum) are only needed at the very end: each thread
+            // keeps its partial through the packed-V phase and the fold rides on that phase's
+            // closing barriers.
+            __syncthreads();   // publishes e and vst
 
             // ---- phase 5: packed V ----------------------------------------------------------
             // lane = (byte column j, slice c of its 8 bit lanes); a wave pass covers TPW tokens
@@ -874,6 +876,20 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                     __builtin_amdgcn_wave_barrier();
                 }
             }
+            // per-wave partial sums of e (and of e * minimum), folded by the output threads below
+            constexpr int kSums = VTOK ? (L::NGRP + 1) * HPB : HPB;
+#pragma unroll
+            for (int h = 0; h < HPB; ++h) {
+                const float x = wave_sum(ls[h]);
+                if (lane == 0) red[wv * kSums + h] = x;
+            }
+            if constexpr (VTOK) {
+#pragma unroll
+                for (int i = 0; i < L::NGRP * HPB; ++i) {
+                    const float x = wave_sum(cma[i]);
+                    if (lane == 0) red[wv * kSums + HPB + i] = x;
+                }
+            }
             __syncthreads();
             V* redv = reinterpret_cast<V*>(regA);  // [wave][PC]
 #pragma unroll
@@ -900,16 +916,20 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                     for (int w = 0; w < kNW; ++w)
                         a += 2.0f * redv[w * L::PC + lane_hi].v[h] + redv[w * L::PC + lane_hi + 1].v[h];
                 }
+                float lh = 0.f;   // sum of e of this thread's head
+#pragma unroll
+                for (int w = 0; w < kNW; ++w) lh += red[w * kSums + h];
                 if constexpr (VTOK) {
-                    o_img = a + fx[L::F_VSZ + (d >> 5) * HPB + h];   // + sum_t e * minimum of the channel's group
+                    float cm = 0.f;   // sum_t e * minimum of the channel's group
+#pragma unroll
+                    for (int w = 0; w < kNW; ++w) cm += red[w * kSums + HPB + (d >> 5) * HPB + h];
+                    o_img = a + cm;
                 } else {
                     const float s = fx[L::F_VSZ + d];
                     const float z = fx[L::F_VSZ + kD + d];
-                    float lh = l_img[0];
-#pragma unroll
-                    for (int k = 1; k < HPB; ++k) lh = (h == k) ? l_img[k] : lh;
                     o_img = s * (a - z * lh);
                 }
+                if (d == 0) stat[4 * HPB + h] = lh;
             }
             __syncthreads();
         }
@@ -918,7 +938,7 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
         for (int h = 0; h < HPB; ++h) {
             if (tid == h) {
                 stat[3 * HPB + h] = m_img[h];
-                stat[4 * HPB + h] = l_img[h];
+                if (n == 0) stat[4 * HPB + h] = 0.f;
             }
         }
         // ---- phase 6: merge / write ---------------------------------------------------------
