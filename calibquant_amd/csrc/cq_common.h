@@ -75,8 +75,8 @@ template <typename DT>
 __device__ __forceinline__ float rnd(float f) { return Cvt<DT>::to_float(Cvt<DT>::from_float(f)); }
 
 // 8 consecutive 16-bit elements (one 16-byte load) -> 8 floats
-template <typename DT>
-__device__ __forceinline__ void unpack8(const uint4& v, float* f) {
+template <typename DT, typename V16>   // V16: uint4 or a native 4 x uint32 vector
+__device__ __forceinline__ void unpack8(const V16& v, float* f) {
     f[0] = Cvt<DT>::lo(v.x); f[1] = Cvt<DT>::hi(v.x);
     f[2] = Cvt<DT>::lo(v.y); f[3] = Cvt<DT>::hi(v.y);
     f[4] = Cvt<DT>::lo(v.z); f[5] = Cvt<DT>::hi(v.z);

@@ -250,6 +250,150 @@ __global__ __launch_bounds__(kQThreads) void emit_kernel(const uint16_t* __restr
     }
 }
 
+// ---- one-pass quantise and pack ------------------------------------------------------------
+// A 1024-thread workgroup owns (batch, head, quarter of the channels): 32 channels = 64 bytes of
+// every token row, T <= 3328 tokens, which is 16 bytes x up to 13 rows per thread - the slice
+// stays in registers between the min/max and the emit, so x is read from HBM once.
+// thread = (row r = tid / 4 of a 256-row pass, 16-byte piece q = tid % 4).
+constexpr int kFThreads = 1024;
+constexpr int kFRows = 13;                  // rows per thread at most (13 x 256 = 12 tiles + thumbnail of 256 tokens)
+constexpr int kFMaxT = kFRows * (kFThreads / 4);
+
+template <typename DT, int BITS, int NR>   // NR: rows per thread (T <= NR * 256)
+__global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* __restrict__ x, QuantGeom g, float clip,
+                                                              uint16_t* __restrict__ scale,
+                                                              uint16_t* __restrict__ zero,
+                                                              uint8_t* __restrict__ codes) {
+    constexpr int L = (1 << BITS) - 1;
+    constexpr float levels = static_cast<float>(L);
+    __shared__ float part[kFThreads / 16][4][16];   // [wave * 4 + row of 16 lanes][piece][min x8, max x8]
+    __shared__ float s_s[32], s_z[32], s_thr[3][32];
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int q4 = tid & 3, row = tid >> 2;
+    // the four quarters of one (batch, head) sit on one XCD (block ids 8 apart), so the four
+    // 4-byte pieces of a packed row meet in one L2
+    const int quarter = (blockIdx.x >> 3) & 3;
+    const int64_t bh = static_cast<int64_t>(blockIdx.x >> 5) * 8 + (blockIdx.x & 7);
+    if (bh >= static_cast<int64_t>(g.B) * g.H) return;
+    const int b = static_cast<int>(bh / g.H), h = static_cast<int>(bh % g.H);
+    const uint16_t* base = x + b * g.sb + h * g.sh + quarter * 32 + q4 * 8;
+
+    typedef uint32_t U4 __attribute__((ext_vector_type(4)));
+    U4 v[NR];
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {   // rows past T re-read row T-1: min / max unchanged, never written
+        const int t = min(i * (kFThreads / 4) + row, g.T - 1);
+        v[i] = *reinterpret_cast<const U4*>(base + t * g.st);
+    }
+    float mn[8], mx[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) { mn[j] = INFINITY; mx[j] = -INFINITY; }
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+        float f[8];
+        unpack8<DT>(v[i], f);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { mn[j] = fminf(mn[j], f[j]); mx[j] = fmaxf(mx[j], f[j]); }
+        __builtin_amdgcn_sched_barrier(0);   // one row at a time: unpacking all rows ahead would not fit the registers
+    }
+    // lanes l, l+4, l+8, l+12 of a row of 16 lanes hold the same channels: two rotations fold them
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        mn[j] = fminf(mn[j], dpp_move<0x124>(mn[j], INFINITY));   // row_ror:4
+        mn[j] = fminf(mn[j], dpp_move<0x128>(mn[j], INFINITY));   // row_ror:8
+        mx[j] = fmaxf(mx[j], dpp_move<0x124>(mx[j], -INFINITY));
+        mx[j] = fmaxf(mx[j], dpp_move<0x128>(mx[j], -INFINITY));
+    }
+    if ((lane & 15) < 4) {
+        float* o = part[wv * 4 + (lane >> 4)][q4];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { o[j] = mn[j]; o[8 + j] = mx[j]; }
+    }
+    __syncthreads();
+    if (tid < 32) {   // channel c of the quarter: fold the 64 partials, run the statistics chain
+        const int c = tid;
+        float a = INFINITY, z = -INFINITY;
+#pragma unroll 4
+        for (int p = 0; p < kFThreads / 16; ++p) {
+            a = fminf(a, part[p][c >> 3][c & 7]);
+            z = fmaxf(z, part[p][c >> 3][8 + (c & 7)]);
+        }
+        const float x_min = rnd<DT>(a * clip);
+        const float x_max = rnd<DT>(z * clip);
+        const float diff = rnd<DT>(x_max - x_min);
+        const float sc = rnd<DT>(diff * __fdiv_rn(1.0f, levels));
+        const float zp = rnd<DT>(__fdiv_rn(-x_min, sc));
+        const int64_t o = bh * g.D + quarter * 32 + c;
+        scale[o] = static_cast<uint16_t>(Cvt<DT>::from_float(sc));
+        zero[o] = static_cast<uint16_t>(Cvt<DT>::from_float(zp));
+        s_s[c] = sc;
+        s_z[c] = zp;
+    }
+    __syncthreads();
+    // thresholds (see the statistics kernel): one 64-ary search per (channel, level) and wave,
+    // three rounds narrow the 2^16 ordered storage values down to one.  The code is a
+    // non-decreasing function of x for every (scale, zero-point) the chain can produce -
+    // also for scale 0 (x / 0 is -inf, NaN, +inf in that order and NaN maps to code 0) and
+    // for NaN statistics (every code 0) - so the search runs for every channel.
+    for (int sid = wv; sid < 32 * L; sid += kFThreads / 64) {
+        const int c = sid / L, k = sid % L + 1;
+        const float sc = s_s[c], zp = s_z[c];
+        float t = NAN;   // stays NaN if no value reaches code k
+        int lo = Keys<DT>::lo - 1, hi = Keys<DT>::hi;   // code(lo) < k (lo may be the virtual floor), answer in (lo, hi]
+        bool reach = true;
+        for (int round = 0; round < 3 && reach; ++round) {
+            const int step = (hi - lo + 63) / 64;
+            const int key = min(lo + (lane + 1) * step, hi);
+            const bool pred = quant_value<DT>(key_value<DT>(key), sc, zp, levels) >= static_cast<float>(k);
+            const unsigned long long m = __ballot(pred);
+            if (m == 0) { reach = false; break; }
+            const int f = __builtin_ctzll(m);
+            hi = min(lo + (f + 1) * step, hi);
+            lo = lo + f * step;
+        }
+        if (reach) t = key_value<DT>(hi);
+        if (lane == 0) s_thr[k - 1][c] = t;
+    }
+    __syncthreads();
+    float th[L][8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int k = 0; k < L; ++k) th[k][j] = s_thr[k][q4 * 8 + j];
+    constexpr int nb = 128 * BITS / 8;   // bytes per packed row
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+        const int t = i * (kFThreads / 4) + row;
+        // (the empty statement keeps the compiler from carrying the unpacked floats of the
+        // min/max pass over to here: that would double the registers the slice needs)
+        asm volatile("" : "+v"(v[i]));
+        float f[8];
+        unpack8<DT>(v[i], f);
+        uint32_t code[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            code[j] = (f[j] >= th[0][j]) ? 1u : 0u;
+            if constexpr (BITS == 2) code[j] += ((f[j] >= th[1][j]) ? 1u : 0u) + ((f[j] >= th[2][j]) ? 1u : 0u);
+        }
+        uint8_t* o = codes + (bh * g.T + min(t, g.T - 1)) * nb + quarter * (nb / 4);
+        if constexpr (BITS == 1) {
+            uint32_t w = 0;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) w |= code[j] << (7 - j);
+            w <<= 8 * q4;
+            w |= static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(w), 0xB1, 0xf, 0xf, true));
+            w |= static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(w), 0x4E, 0xf, 0xf, true));
+            if (q4 == 0 && t < g.T) *reinterpret_cast<uint32_t*>(o) = w;
+        } else {
+            const uint32_t b0 = (code[0] << 6) | (code[1] << 4) | (code[2] << 2) | code[3];
+            const uint32_t b1 = (code[4] << 6) | (code[5] << 4) | (code[6] << 2) | code[7];
+            const uint32_t half = b0 | (b1 << 8);
+            const uint32_t other = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(half), 0xB1, 0xf, 0xf, true));
+            if ((q4 & 1) == 0 && t < g.T) reinterpret_cast<uint32_t*>(o)[q4 >> 1] = half | (other << 16);
+        }
+    }
+}
+
 template <typename DT>
 static int run_quant(const void* x, QuantGeom g, int bits, float clip, uint8_t* codes, void* xq, void* scale,
                      void* zero, float* ws, hipStream_t st) {
@@ -257,6 +401,21 @@ static int run_quant(const void* x, QuantGeom g, int bits, float clip, uint8_t* 
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     uint16_t* sp = static_cast<uint16_t*>(scale);
     uint16_t* zp = static_cast<uint16_t*>(zero);
+    if (!xq && g.D == 128 && g.T <= kFMaxT && (reinterpret_cast<uintptr_t>(codes) & 3u) == 0) {
+        // x fits a workgroup's registers slice by slice: one pass
+        const int64_t bh8 = (static_cast<int64_t>(g.B) * g.H + 7) / 8;
+        const dim3 fgrid(static_cast<unsigned>(bh8 * 32));
+        const int nr = (g.T + kFThreads / 4 - 1) / (kFThreads / 4);
+#define CQ_FUSED(B_, N_) hipLaunchKernelGGL((fused_pack_kernel<DT, B_, N_>), fgrid, dim3(kFThreads), 0, st, xp, g, clip, sp, zp, codes)
+        if (bits == 1) {
+            if (nr <= 4) CQ_FUSED(1, 4); else if (nr <= 8) CQ_FUSED(1, 8); else CQ_FUSED(1, 13);
+        } else {
+            if (nr <= 4) CQ_FUSED(2, 4); else if (nr <= 8) CQ_FUSED(2, 8); else CQ_FUSED(2, 13);
+        }
+#undef CQ_FUSED
+        CQ_LAUNCH_CHECK();
+        return CQ_OK;
+    }
     hipLaunchKernelGGL(minmax_partial_kernel<DT>, grid, dim3(kQThreads), 0, st, xp, g, ws);
     CQ_LAUNCH_CHECK();
     const float levels = static_cast<float>((1 << bits) - 1);

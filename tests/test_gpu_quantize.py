@@ -16,7 +16,8 @@ def ops():
     return ops
 
 
-SHAPES = [(2, 257, 3, 128), (1, 1, 2, 128), (3, 63, 1, 64), (1, 1000, 2, 256), (2, 3328, 8, 128)]
+SHAPES = [(2, 257, 3, 128), (1, 1, 2, 128), (3, 63, 1, 64), (1, 1000, 2, 256), (2, 3328, 8, 128),
+          (1, 1500, 1, 128), (1, 2100, 2, 128), (1, 5000, 2, 128)]   # one-pass kernel row counts; beyond its reach
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp16"])
