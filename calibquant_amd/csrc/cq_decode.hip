@@ -3,10 +3,12 @@
 // One 1024-thread workgroup owns one (batch, kv-head, head-group, token-chunk)
 // unit and runs the whole step for HPB query heads that share the kv-head:
 //
-//   loads    every global load the unit needs first (packed K rows, the first
-//            block of packed V rows, the first tile of residual K/V rows) is
-//            issued at kernel entry into registers, so HBM latency overlaps
-//            the table build instead of stalling each phase in turn.
+//   loads    the packed K rows are requested at kernel entry, the first block of
+//            packed V rows behind them (half before the logits, half as the K
+//            registers free up), the first tile of residual K/V rows when the
+//            packed-V phase ends: each stream is in flight while the phase before
+//            its consumer runs, and no phase starts behind a queue of requests
+//            it does not need.
 //   K side   q.s_k is folded into a byte-indexed partial-sum table in LDS
 //            (one entry per byte position and byte value, HPB floats wide,
 //            zero-point folded in).  A token's logits are NB table look-ups
@@ -19,7 +21,7 @@
 //            column in one dword), a 4-byte dot product turns each bit lane of the
 //            column into a table offset, and the lane adds that table entry.  Scale /
 //            zero-point are applied once at the end.
-//   residual the full-precision rows run as an online-softmax flash-decode in
+//   residual the full-precision rows run last as an online-softmax flash-decode in
 //            the same workgroup (packed dot2 for q.K) and are merged at the end.
 //
 // When the chunk does not cover all T tokens (long context or small batch)
@@ -234,9 +236,9 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
     const int npad = (n + L::TPW - 1) / L::TPW * L::TPW;
     const float inv_sqrt_d = 0.08838834764831845f;  // 1/sqrt(128)
 
-    // ---- entry: put the unit's global loads in flight.  The vector-memory counter is
-    // in order, so the few elements phase 0 needs are requested first and the bulk
-    // streams (packed K, packed V, residual tile) behind them.
+    // ---- entry: put the unit's first global loads in flight.  The vector-memory counter is
+    // in order, so the few elements phase 0 needs are requested first and the packed K rows
+    // behind them; packed V rows and the residual tile follow later (see the file header).
     // Loads are unconditional with clamped (always valid) addresses: no divergent
     // control flow around them, so the compiler can wait on exactly the counter value
     // each consumer needs.
@@ -284,16 +286,11 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
             v2[rep] = *reinterpret_cast<const uint4*>(vbp + r2 * rs_r + ds * 8);
         }
     };
-    if constexpr (!MINMAX_ONLY) {
-        load_res_k(0, rk);
-        load_res_v(0, rv);
-    }
     uint4 kc[L::KR][BITS];
 #pragma unroll
-    for (int r = 0; r < L::KR; ++r) {   // first half now, second half once the residual phase is done
+    for (int r = 0; r < L::KR; ++r) {
 #pragma unroll
-        for (int i = 0; i < BITS; ++i)
-            if (r * BITS + i < kPF / 2) kc[r][i] = ckp[min((tid + r * kNT) * BITS + i, last_u)];
+        for (int i = 0; i < BITS; ++i) kc[r][i] = ckp[min((tid + r * kNT) * BITS + i, last_u)];
     }
 
     // ---- phase 0: q, per-bit weights ---------------------------------------------------
@@ -326,114 +323,6 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
 
     float* stat = fx + L::F_STAT;   // [alpha | m_res | l_res | m_img | l_img][HPB]
     float o_res = 0.f;
-    if constexpr (!MINMAX_ONLY) {
-        // ---- phase 1: full-precision residual rows, online softmax.  Runs first: its rows
-        // were requested first, and the packed K rows keep streaming in meanwhile.
-#pragma unroll
-        for (int h = 0; h < HPB; ++h) {
-            if (tid == h) {
-                stat[HPB + h] = -INFINITY;
-                stat[2 * HPB + h] = 0.f;
-            }
-        }
-        if (do_res) {
-            float m_run = -INFINITY, l_run = 0.f;
-            float* sres = fx + L::F_SRES;
-            float* pres = fx + L::F_PRES;
-            // raw 16-bit q, [head][kD], read per head as two 16-byte LDS loads
-            const uint4* q128 = reinterpret_cast<const uint4*>(fx + L::F_QRAW);
-            float accv[8][HPB];
-#pragma unroll
-            for (int k = 0; k < 8; ++k)
-#pragma unroll
-                for (int h = 0; h < HPB; ++h) accv[k][h] = 0.f;
-            const float* mk = g.mask ? g.mask + b * g.mask_sb : nullptr;
-
-            for (int r0 = 0; r0 < R; r0 += kResTile) {
-                const bool more = r0 + kResTile < R;
-                const int r = r0 + krow;
-                float dot[HPB];
-#pragma unroll
-                for (int h = 0; h < HPB; ++h) {
-                    const uint4 qa = q128[h * (kD / 8) + l8];
-                    const uint4 qb = q128[h * (kD / 8) + 8 + l8];
-                    float a = 0.f;
-                    a = dot2<DT>(qa.x, rk[0].x, a); a = dot2<DT>(qa.y, rk[0].y, a);
-                    a = dot2<DT>(qa.z, rk[0].z, a); a = dot2<DT>(qa.w, rk[0].w, a);
-                    a = dot2<DT>(qb.x, rk[1].x, a); a = dot2<DT>(qb.y, rk[1].y, a);
-                    a = dot2<DT>(qb.z, rk[1].z, a); a = dot2<DT>(qb.w, rk[1].w, a);
-                    dot[h] = oct_reduce(a, OpSum(), 0.f) * inv_sqrt_d;
-                }
-                if (more) load_res_k(r0 + kResTile, rk);   // next tile's K slice, in place
-                if (l8 == 0) {
-                    float mv = 0.f;
-                    if (mk && r < R) mv = mk[r < g.S ? r : g.T + r];
-#pragma unroll
-                    for (int h = 0; h < HPB; ++h) sres[krow * HPB + h] = (r < R) ? dot[h] + mv : -INFINITY;
-                }
-                __syncthreads();
-                if (wv < HPB) {   // wave h keeps the running softmax state of head h
-                    const int h = wv;
-                    const float s0 = sres[lane * HPB + h];
-                    const float s1 = sres[(lane + 64) * HPB + h];
-                    const float mnew = fmaxf(m_run, wave_max(fmaxf(s0, s1)));
-                    const bool dead = (mnew == -INFINITY);
-                    const float p0 = dead ? 0.f : __expf(s0 - mnew);
-                    const float p1 = dead ? 0.f : __expf(s1 - mnew);
-                    const float al = dead ? 1.0f : __expf(m_run - mnew);
-                    l_run = l_run * al + wave_sum(p0 + p1);
-                    m_run = mnew;
-                    pres[lane * HPB + h] = p0;
-                    pres[(lane + 64) * HPB + h] = p1;
-                    if (lane == 0) { stat[h] = al; stat[HPB + h] = m_run; stat[2 * HPB + h] = l_run; }
-                }
-                __syncthreads();
-                float alpha[HPB];
-#pragma unroll
-                for (int h = 0; h < HPB; ++h) alpha[h] = stat[h];
-#pragma unroll
-                for (int rep = 0; rep < 2; ++rep) {
-                    const int rr = rslot + rep * (kResTile / 2);
-                    float f[8];
-                    unpack8<DT>(rv[rep], f);
-                    const V p = reinterpret_cast<const V*>(pres)[rr];   // 0 for rows past R
-#pragma unroll
-                    for (int k = 0; k < 8; ++k)
-#pragma unroll
-                        for (int h = 0; h < HPB; ++h)
-                            accv[k][h] = ((rep == 0 && r0 > 0) ? accv[k][h] * alpha[h] : accv[k][h]) + p.v[h] * f[k];
-                }
-                if (more) load_res_v(r0 + kResTile, rv);   // next tile's V slices, in place
-            }
-            // fold the row slots: 4 per wave (lane bits 4,5), then the waves
-#pragma unroll
-            for (int k = 0; k < 8; ++k)
-#pragma unroll
-                for (int h = 0; h < HPB; ++h) accv[k][h] = quad_reduce(accv[k][h], OpSum(), 0.f);
-            __syncthreads();
-            float* red2 = reinterpret_cast<float*>(regA);  // [wave][kD][HPB]
-            if ((lane & 3) == 0) {
-#pragma unroll
-                for (int k = 0; k < 8; ++k)
-#pragma unroll
-                    for (int h = 0; h < HPB; ++h) red2[(wv * kD + ds * 8 + k) * HPB + h] = accv[k][h];
-            }
-            __syncthreads();
-            if (tid < HPB * kD) {
-                const int h = tid / kD, d = tid % kD;
-#pragma unroll
-                for (int w = 0; w < kNW; ++w) o_res += red2[(w * kD + d) * HPB + h];
-            }
-        }
-
-    }
-
-#pragma unroll
-    for (int r = 0; r < L::KR; ++r) {
-#pragma unroll
-        for (int i = 0; i < BITS; ++i)
-            if (r * BITS + i >= kPF / 2) kc[r][i] = ckp[min((tid + r * kNT) * BITS + i, last_u)];
-    }
     float mn[HPB], mx[HPB];
 #pragma unroll
     for (int h = 0; h < HPB; ++h) { mn[h] = INFINITY; mx[h] = -INFINITY; }
@@ -876,6 +765,8 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                     __builtin_amdgcn_wave_barrier();
                 }
             }
+            load_res_k(0, rk);   // first residual tile: in flight during the fold below
+            load_res_v(0, rv);
             // per-wave partial sums of e (and of e * minimum), folded by the output threads below
             constexpr int kSums = VTOK ? (L::NGRP + 1) * HPB : HPB;
 #pragma unroll
@@ -934,6 +825,109 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
             __syncthreads();
         }
 
+        if (n == 0) {
+            load_res_k(0, rk);
+            load_res_v(0, rv);
+        }
+        // ---- phase 6: full-precision residual rows, online softmax.  Runs last: its first
+        // tile is requested when the packed-V phase ends and arrives during that phase's fold.
+#pragma unroll
+        for (int h = 0; h < HPB; ++h) {
+            if (tid == h) {
+                stat[HPB + h] = -INFINITY;
+                stat[2 * HPB + h] = 0.f;
+            }
+        }
+        if (do_res) {
+            float m_run = -INFINITY, l_run = 0.f;
+            float* sres = fx + L::F_SRES;
+            float* pres = fx + L::F_PRES;
+            // raw 16-bit q, [head][kD], read per head as two 16-byte LDS loads
+            const uint4* q128 = reinterpret_cast<const uint4*>(fx + L::F_QRAW);
+            float accv[8][HPB];
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+#pragma unroll
+                for (int h = 0; h < HPB; ++h) accv[k][h] = 0.f;
+            const float* mk = g.mask ? g.mask + b * g.mask_sb : nullptr;
+
+            for (int r0 = 0; r0 < R; r0 += kResTile) {
+                const bool more = r0 + kResTile < R;
+                const int r = r0 + krow;
+                float dot[HPB];
+#pragma unroll
+                for (int h = 0; h < HPB; ++h) {
+                    const uint4 qa = q128[h * (kD / 8) + l8];
+                    const uint4 qb = q128[h * (kD / 8) + 8 + l8];
+                    float a = 0.f;
+                    a = dot2<DT>(qa.x, rk[0].x, a); a = dot2<DT>(qa.y, rk[0].y, a);
+                    a = dot2<DT>(qa.z, rk[0].z, a); a = dot2<DT>(qa.w, rk[0].w, a);
+                    a = dot2<DT>(qb.x, rk[1].x, a); a = dot2<DT>(qb.y, rk[1].y, a);
+                    a = dot2<DT>(qb.z, rk[1].z, a); a = dot2<DT>(qb.w, rk[1].w, a);
+                    dot[h] = oct_reduce(a, OpSum(), 0.f) * inv_sqrt_d;
+                }
+                if (more) load_res_k(r0 + kResTile, rk);   // next tile's K slice, in place
+                if (l8 == 0) {
+                    float mv = 0.f;
+                    if (mk && r < R) mv = mk[r < g.S ? r : g.T + r];
+#pragma unroll
+                    for (int h = 0; h < HPB; ++h) sres[krow * HPB + h] = (r < R) ? dot[h] + mv : -INFINITY;
+                }
+                __syncthreads();
+                if (wv < HPB) {   // wave h keeps the running softmax state of head h
+                    const int h = wv;
+                    const float s0 = sres[lane * HPB + h];
+                    const float s1 = sres[(lane + 64) * HPB + h];
+                    const float mnew = fmaxf(m_run, wave_max(fmaxf(s0, s1)));
+                    const bool dead = (mnew == -INFINITY);
+                    const float p0 = dead ? 0.f : __expf(s0 - mnew);
+                    const float p1 = dead ? 0.f : __expf(s1 - mnew);
+                    const float al = dead ? 1.0f : __expf(m_run - mnew);
+                    l_run = l_run * al + wave_sum(p0 + p1);
+                    m_run = mnew;
+                    pres[lane * HPB + h] = p0;
+                    pres[(lane + 64) * HPB + h] = p1;
+                    if (lane == 0) { stat[h] = al; stat[HPB + h] = m_run; stat[2 * HPB + h] = l_run; }
+                }
+                __syncthreads();
+                float alpha[HPB];
+#pragma unroll
+                for (int h = 0; h < HPB; ++h) alpha[h] = stat[h];
+#pragma unroll
+                for (int rep = 0; rep < 2; ++rep) {
+                    const int rr = rslot + rep * (kResTile / 2);
+                    float f[8];
+                    unpack8<DT>(rv[rep], f);
+                    const V p = reinterpret_cast<const V*>(pres)[rr];   // 0 for rows past R
+#pragma unroll
+                    for (int k = 0; k < 8; ++k)
+#pragma unroll
+                        for (int h = 0; h < HPB; ++h)
+                            accv[k][h] = ((rep == 0 && r0 > 0) ? accv[k][h] * alpha[h] : accv[k][h]) + p.v[h] * f[k];
+                }
+                if (more) load_res_v(r0 + kResTile, rv);   // next tile's V slices, in place
+            }
+            // fold the row slots: 4 per wave (lane bits 4,5), then the waves
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+#pragma unroll
+                for (int h = 0; h < HPB; ++h) accv[k][h] = quad_reduce(accv[k][h], OpSum(), 0.f);
+            __syncthreads();
+            float* red2 = reinterpret_cast<float*>(regA);  // [wave][kD][HPB]
+            if ((lane & 3) == 0) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+#pragma unroll
+                    for (int h = 0; h < HPB; ++h) red2[(wv * kD + ds * 8 + k) * HPB + h] = accv[k][h];
+            }
+            __syncthreads();
+            if (tid < HPB * kD) {
+                const int h = tid / kD, d = tid % kD;
+#pragma unroll
+                for (int w = 0; w < kNW; ++w) o_res += red2[(w * kD + d) * HPB + h];
+            }
+        }
+
 #pragma unroll
         for (int h = 0; h < HPB; ++h) {
             if (tid == h) {
@@ -941,7 +935,7 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                 if (n == 0) stat[4 * HPB + h] = 0.f;
             }
         }
-        // ---- phase 6: merge / write ---------------------------------------------------------
+        // ---- phase 7: merge / write ---------------------------------------------------------
         __syncthreads();
         if (tid < HPB * kD) {
             const int h = tid / kD, d = tid % kD;
