@@ -193,6 +193,16 @@ template <int N> __device__ __forceinline__ Words<N> lds_words(uint32_t addr) {
     return r;
 }
 
+// N floats at an absolute LDS byte address.
+template <int N> __device__ __forceinline__ Vec<N> lds_floats(uint32_t addr) {
+    typedef float VT __attribute__((ext_vector_type(N)));
+    const VT v = *(const __attribute__((address_space(3))) VT*)(static_cast<uintptr_t>(addr));
+    Vec<N> r;
+#pragma unroll
+    for (int k = 0; k < N; ++k) r.v[k] = v[k];
+    return r;
+}
+
 __device__ __forceinline__ uint32_t pack_f16(float a, float b) {
     f16x2_t h = {static_cast<_Float16>(a), static_cast<_Float16>(b)};   // round to nearest even
     return __builtin_bit_cast(uint32_t, h);
@@ -428,7 +438,10 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                     V cur;
                     if constexpr (kPermAddr) {
                         const uint32_t sel = static_cast<uint32_t>(k & 3) | (static_cast<uint32_t>(4 + (k & 3)) << 8) | 0x0c0c0000u;
-                        cur = *reinterpret_cast<const V*>(ktab_b + __builtin_amdgcn_perm(wds[k >> 2], pofs4[k >> 2], sel));
+                        // The kernel's only LDS object is the dynamic array, so it starts at LDS
+                        // address 0 and the K table with it (the host checks that the kernel has no
+                        // static LDS before the first launch): the permute result is the address.
+                        cur = lds_floats<HPB>(__builtin_amdgcn_perm(wds[k >> 2], pofs4[k >> 2], sel));
                     } else {
                         const uint32_t byte = (wds[k >> 2] >> (8 * (k & 3))) & 0xffu;
                         cur = *reinterpret_cast<const V*>(ktab_b + byte * (NB * L::ESZ) + pofs[k]);
@@ -1051,6 +1064,12 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
     CQ_HIP_CHECK(hipGetDevice(&dev));
     const uint32_t bit = 1u << (dev & 31);
     if (!(attr_done.load(std::memory_order_acquire) & bit)) {
+        // the K look-ups address the table absolutely: the dynamic LDS array must start at 0
+        hipFuncAttributes fa;
+        CQ_HIP_CHECK(hipFuncGetAttributes(&fa, reinterpret_cast<const void*>(kmain)));
+        if (fa.sharedSizeBytes != 0) return CQ_ERR_LAUNCH;
+        CQ_HIP_CHECK(hipFuncGetAttributes(&fa, reinterpret_cast<const void*>(kmm)));
+        if (fa.sharedSizeBytes != 0) return CQ_ERR_LAUNCH;
         CQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kmain),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax));
         CQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kmm),
