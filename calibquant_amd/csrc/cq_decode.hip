@@ -48,6 +48,19 @@ template <int N> struct alignas(N * 4) Vec { float v[N]; };
 // native 16-byte vector: copies are single vector moves (HIP's uint4 struct copies lower to memcpy)
 typedef uint32_t U4 __attribute__((ext_vector_type(4)));
 
+// Division of block indices (< 2^31) by a small run-time constant without the integer-division
+// expansion: q = (mulhi(n, mul) + n) >> shift, with mul and shift worked out on the host.
+struct FastDiv {
+    uint32_t mul, shift, div;
+    __host__ void set(uint32_t d) {
+        div = d;
+        shift = 0;
+        while ((1u << shift) < d) ++shift;
+        mul = static_cast<uint32_t>(((static_cast<uint64_t>(1) << 32) * ((static_cast<uint64_t>(1) << shift) - d)) / d + 1);
+    }
+    __device__ __forceinline__ uint32_t quot(uint32_t n) const { return (__umulhi(n, mul) + n) >> shift; }
+};
+
 struct DecodeGeom {
     const void* q;
     const uint8_t* ck;
@@ -66,6 +79,8 @@ struct DecodeGeom {
     int calib;
     float off_max, off_min;
     int cap;      // logits capacity of the LDS layout, tokens
+    FastDiv d_ng, d_nx, d_hkv;   // divisors of the unit decomposition: head groups, chunks (+ residual unit), kv heads
+    int G;        // query heads per kv head
     float one;    // 1.0f, opaque to the compiler: keeps f16 -> f32 accumulation in one mixed-precision FMA
 };
 
@@ -227,14 +242,16 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wv = tid >> 6;
-    const int G = g.Hq / g.Hkv;
-    const int NG = G / HPB;
+    const int G = g.G;
 
-    int vb = virtual_block_id();
-    const int hg = vb % NG; vb /= NG;
-    const int split = vb % g.nx; vb /= g.nx;
-    const int hkv = vb % g.Hkv;
-    const int b = vb / g.Hkv;
+    uint32_t vb = static_cast<uint32_t>(virtual_block_id());
+    uint32_t qn = g.d_ng.quot(vb);
+    const int hg = static_cast<int>(vb - qn * g.d_ng.div); vb = qn;
+    qn = g.d_nx.quot(vb);
+    const int split = static_cast<int>(vb - qn * g.d_nx.div); vb = qn;
+    qn = g.d_hkv.quot(vb);
+    const int hkv = static_cast<int>(vb - qn * g.d_hkv.div);
+    const int b = static_cast<int>(qn);
     const int hq0 = hkv * G + hg * HPB;
     const int64_t bh = static_cast<int64_t>(b) * g.Hkv + hkv;
 
@@ -246,9 +263,8 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
     const int npad = (n + L::TPW - 1) / L::TPW * L::TPW;
     const float inv_sqrt_d = 0.08838834764831845f;  // 1/sqrt(128)
 
-    // ---- entry: put the unit's first global loads in flight.  The vector-memory counter is
-    // in order, so the few elements phase 0 needs are requested first and the packed K rows
-    // behind them; packed V rows and the residual tile follow later (see the file header).
+    // ---- entry: the few elements phase 0 needs are requested first; the packed K rows follow
+    // phase 0, packed V rows and the residual tile later still (see the file header).
     // Loads are unconditional with clamped (always valid) addresses: no divergent
     // control flow around them, so the compiler can wait on exactly the counter value
     // each consumer needs.
@@ -296,12 +312,6 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
             v2[rep] = *reinterpret_cast<const uint4*>(vbp + r2 * rs_r + ds * 8);
         }
     };
-    uint4 kc[L::KR][BITS];
-#pragma unroll
-    for (int r = 0; r < L::KR; ++r) {
-#pragma unroll
-        for (int i = 0; i < BITS; ++i) kc[r][i] = ckp[min((tid + r * kNT) * BITS + i, last_u)];
-    }
 
     // ---- phase 0: q, per-bit weights ---------------------------------------------------
     if (tid < HPB * kD) {
@@ -314,7 +324,11 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
             const float s = Cvt<DT>::to_float(s_raw);
             const float z = Cvt<DT>::to_float(z_raw);
             const float qs = qv * s;
-            qsz[h * kD + d] = qs * z;
+            // zero-point term of the byte position: sum of q s z over the channels of one byte
+            // (consecutive lanes), kept [byte position][head]
+            constexpr int cpb0 = 8 / BITS;
+            const float zsum = (cpb0 == 8) ? oct_reduce(qs * z, OpSum(), 0.f) : quad_reduce(qs * z, OpSum(), 0.f);
+            if (d % cpb0 == 0) qsz[(d / cpb0) * HPB + h] = zsum;
             if constexpr (BITS == 1) {
                 wbit[((d >> 3) * 8 + (7 - (d & 7))) * HPB + h] = qs;
             } else {
@@ -328,6 +342,15 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
         const int d = tid - (kNT - kD);
         fx[L::F_VSZ + d] = Cvt<DT>::to_float(s_raw);
         fx[L::F_VSZ + kD + d] = Cvt<DT>::to_float(z_raw);
+    }
+    // The packed K rows are requested only now: a wave that has to queue 64 KB of requests
+    // first gets to phase 0 thousands of cycles later, and the table build below covers
+    // their latency anyway.
+    uint4 kc[L::KR][BITS];
+#pragma unroll
+    for (int r = 0; r < L::KR; ++r) {
+#pragma unroll
+        for (int i = 0; i < BITS; ++i) kc[r][i] = ckp[min((tid + r * kNT) * BITS + i, last_u)];
     }
     __syncthreads();
 
@@ -355,17 +378,10 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
         for (int e = tid; e < NB * 32; e += kNT) {
             const int j = e % NB, half = (e / NB) >> 4, v = (e / NB) & 15;
             const V* wb = reinterpret_cast<const V*>(wbit) + j * 8 + half * 4;
-            constexpr int cpb = 8 / BITS;
             V acc;
+            const V zs = reinterpret_cast<const V*>(qsz)[j];
 #pragma unroll
-            for (int h = 0; h < HPB; ++h) {
-                float zs = 0.f;
-                if (half) {
-#pragma unroll
-                    for (int i = 0; i < cpb; ++i) zs += qsz[h * kD + j * cpb + i];
-                }
-                acc.v[h] = -zs;
-            }
+            for (int h = 0; h < HPB; ++h) acc.v[h] = half ? -zs.v[h] : 0.f;
 #pragma unroll
             for (int bt = 0; bt < 4; ++bt) {
                 const V w4 = wb[bt];
@@ -1076,15 +1092,21 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
                                          hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax));
         attr_done.fetch_or(bit, std::memory_order_release);
     }
+    DecodeGeom gm = g;
+    gm.G = G;
+    gm.d_ng.set(static_cast<uint32_t>(G / HPB));
+    gm.d_nx.set(static_cast<uint32_t>(g.nx));
+    gm.d_hkv.set(static_cast<uint32_t>(g.Hkv));
     if (g.nsplit > 1) {
-        DecodeGeom g1 = g;
+        DecodeGeom g1 = gm;
         g1.nx = g.nsplit;  // the min/max pass has no residual unit
+        g1.d_nx.set(static_cast<uint32_t>(g.nsplit));
         g1.cap = 0;        // ... and keeps no logits
         const int lds_mm = Lay<BITS, HPB, false>::lds_bytes(0);
         hipLaunchKernelGGL(kmm, dim3(units * g.nsplit), dim3(kNT), lds_mm, st, g1);
         CQ_LAUNCH_CHECK();
     }
-    hipLaunchKernelGGL(kmain, dim3(units * g.nx), dim3(kNT), p.lds, st, g);
+    hipLaunchKernelGGL(kmain, dim3(units * g.nx), dim3(kNT), p.lds, st, gm);
     CQ_LAUNCH_CHECK();
     if (g.nsplit > 1) {
         hipLaunchKernelGGL(merge_kernel<DT>, dim3(static_cast<unsigned>(g.B) * g.Hq), dim3(kD), 0, st, g.part, g.nx,
