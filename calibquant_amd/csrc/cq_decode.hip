@@ -540,24 +540,26 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
             // (ordered by the barriers of block_reduce).  Layout: [unit of TPW tokens]
             // [byte column][token], so the 4 bytes that the 4 tokens of a group have in one
             // column form one dword.  A quad of lanes holds a group (tokens are
-            // lane-consecutive): each lane gathers, for 4 of the 16 columns of its 16-byte
-            // piece, the 4 tokens' bytes with quad broadcasts and byte permutes.
+            // lane-consecutive): per dword of its 16-byte piece the quad transposes a 4 x 4 byte
+            // block in two exchange steps (lane ^ 1, then lane ^ 2), a byte permute after each,
+            // and lane i ends up with the 4 tokens' bytes of column 4 q + i.
             unsigned char* vst = regA + L::WTAB;
             const int qi = lane & 3;
-            const uint32_t sel_pair = static_cast<uint32_t>(qi) | (static_cast<uint32_t>(4 + qi) << 8) | 0x0c0c0000u;
+            // step 1, operands (partner, own): bytes qi and qi ^ 2 of the even and of the odd lane
+            const uint32_t b0 = static_cast<uint32_t>(qi), b2 = static_cast<uint32_t>(qi ^ 2);
+            const uint32_t sel1 = (qi & 1) ? ((4 + b0) | (b0 << 8) | ((4 + b2) << 16) | (b2 << 24))
+                                           : (b0 | ((4 + b0) << 8) | (b2 << 16) | ((4 + b2) << 24));
+            // step 2, operands (partner, own): own low half and the partner's high half, pair 0 first
+            const uint32_t sel2 = (qi & 2) ? 0x01000706u : 0x07060100u;
             auto stage_piece = [&](U4 c, int tok, int piece, bool write) {
                 const uint32_t w[4] = {c.x, c.y, c.z, c.w};
                 const int base = ((tok / L::TPW) * NB + 16 * piece + qi) * L::TPW + ((tok % L::TPW) & ~3);
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    const int wi = static_cast<int>(w[q]);
-                    const uint32_t x0 = __builtin_amdgcn_mov_dpp(wi, 0x00, 0xf, 0xf, true);
-                    const uint32_t x1 = __builtin_amdgcn_mov_dpp(wi, 0x55, 0xf, 0xf, true);
-                    const uint32_t x2 = __builtin_amdgcn_mov_dpp(wi, 0xAA, 0xf, 0xf, true);
-                    const uint32_t x3 = __builtin_amdgcn_mov_dpp(wi, 0xFF, 0xf, 0xf, true);
-                    const uint32_t lo = __builtin_amdgcn_perm(x1, x0, sel_pair);
-                    const uint32_t hi = __builtin_amdgcn_perm(x3, x2, sel_pair);
-                    const uint32_t t4 = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+                    const uint32_t p1 = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(w[q]), 0xB1, 0xf, 0xf, true));
+                    const uint32_t a = __builtin_amdgcn_perm(p1, w[q], sel1);
+                    const uint32_t p2 = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(a), 0x4E, 0xf, 0xf, true));
+                    const uint32_t t4 = __builtin_amdgcn_perm(p2, a, sel2);
                     if (write) *reinterpret_cast<uint32_t*>(vst + base + 4 * q * L::TPW) = t4;
                 }
             };
