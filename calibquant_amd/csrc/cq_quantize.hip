@@ -470,6 +470,9 @@ static int quant_entry(const void* x, int dtype, int B, int T, int H, int D, int
 // IEEE division), 32/BITS codes per int32 word with the first code in the lowest bits.
 // 16 lanes cover a row of 128 channels with one 16-byte load each; the four lanes of a
 // quad are one group.  One pass over x.
+template <typename DT> struct BF16Like { static constexpr bool value = false; };
+template <> struct BF16Like<BF16> { static constexpr bool value = true; };
+
 template <typename DT, int BITS>
 __global__ __launch_bounds__(kQThreads) void token_pack_kernel(const uint16_t* __restrict__ x, QuantGeom g,
                                                                int32_t* __restrict__ words,
@@ -494,13 +497,28 @@ __global__ __launch_bounds__(kQThreads) void token_pack_kernel(const uint16_t* _
         mn = quad_reduce(mn, OpMin(), INFINITY);
         mx = quad_reduce(mx, OpMax(), -INFINITY);
         const float s = rnd<DT>(rnd<DT>(mx - mn) * inv_levels);
+        // bf16: the code steps up where y = bf16(fp32(d / s)), d = bf16(x - min), crosses
+        // 0.5 (exclusive), 1.5 (inclusive), 2.5 (exclusive) under round-half-even, i.e. where
+        // fp32(d / s) crosses the midpoint m to the neighbouring bf16 value.  d and s have 8
+        // significant bits and m at most 10, so s * m is exact in fp32 and d / s is either
+        // exactly m or further from it than fp32 rounding can move it: the comparison
+        // d > s * m (or >=) decides exactly what the division would, without dividing.
+        const bool by_compare = BF16Like<DT>::value && s > 0.0f && s < INFINITY;
+        const float m1 = s * (0.5f + 0.001953125f);      // 0.5 + 2^-9
+        const float m2 = s * (1.5f - 0.00390625f);       // 1.5 - 2^-8
+        const float m3 = s * (2.5f + 0.0078125f);        // 2.5 + 2^-7
         uint32_t packed = 0;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            float y = rnd<DT>(f[i] - mn);
-            y = rnd<DT>(__fdiv_rn(y, s));
+            const float d = rnd<DT>(f[i] - mn);
             uint32_t code = 0;
-            if (y == y) code = static_cast<uint32_t>(rintf(fminf(fmaxf(y, 0.0f), levels)));
+            if (by_compare) {
+                code = (d > m1) ? 1u : 0u;
+                if constexpr (BITS == 2) code += ((d >= m2) ? 1u : 0u) + ((d > m3) ? 1u : 0u);
+            } else {
+                const float y = rnd<DT>(__fdiv_rn(d, s));
+                if (y == y) code = static_cast<uint32_t>(rintf(fminf(fmaxf(y, 0.0f), levels)));
+            }
             packed |= code << (BITS * i);
         }
         const int64_t gidx = row * (g.D / 32) + grp;
