@@ -39,12 +39,9 @@ struct FP16 {};
 
 __device__ __forceinline__ float bf16_bits_to_float(uint32_t h) { return __uint_as_float(h << 16); }
 
-// fp32 -> bf16 bits, round to nearest even, NaN kept quiet.
+// fp32 -> bf16 bits, round to nearest even (the hardware conversion of gfx950).
 __device__ __forceinline__ uint32_t float_to_bf16_bits(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return u >> 16;
+    return __builtin_bit_cast(unsigned short, static_cast<__bf16>(f));
 }
 
 __device__ __forceinline__ float fp16_bits_to_float(uint32_t h) {
