@@ -29,7 +29,11 @@ Pinning status (what each function is checked against in tests/):
   decode_attention_refchain   informational mixed-precision chain; its
                         rounding sequence follows the reference text but
                         no reference-held vector exists for it: parity unpinned
-  kivi_quantize_pack / kivi_pv   closed form + little-endian word packing pinned
+  kivi_quantize_pack / kivi_pv   closed form + little-endian word packing
+                        (numpy.packbits bitorder='little' at b=1), group
+                        min / range, midpoint rule                       pinned
+  decode_attention(v_token_group)   python-loop brute force on explicitly
+                        dequantised scale*code + minimum values          pinned
 """
 from __future__ import annotations
 

@@ -125,3 +125,33 @@ def test_rope_append_equals_the_torch_op_chain_bit_for_bit(dtype, heads):
     ops.RopeAppendCall(qkv, cos, sin, pos, q_out, kwin, vwin, row).run()
     torch.cuda.synchronize()
     assert not kwin.any() and not vwin.any()
+
+
+def test_rope_append_full_batch_and_replay_by_device_counters():
+    """Batch 64 at the 8B head layout: the launch prepared once follows the device-side row and
+    position counters, as a recorded decode step needs."""
+    from calibquant_amd import ops, patch_internvl as pi
+    Hq, Hkv, G, D, B, cap, rows = 32, 8, 4, 128, 64, 8, 4000
+    torch.manual_seed(6)
+    t = torch.arange(rows, device="cuda", dtype=torch.float32)
+    inv = 1.0 / (1e6 ** (torch.arange(0, D, 2, device="cuda").float() / D))
+    emb = torch.cat([torch.outer(t, inv)] * 2, dim=-1)
+    cos, sin = emb.cos().to(torch.bfloat16), emb.sin().to(torch.bfloat16)
+    qkv = torch.empty(B, (Hq + 2 * Hkv) * D, device="cuda", dtype=torch.bfloat16)
+    pos = torch.full((B, 1), 3392, device="cuda", dtype=torch.long)
+    row = torch.zeros(1, device="cuda", dtype=torch.long)
+    kwin = torch.zeros(B, Hkv, cap, D, device="cuda", dtype=torch.bfloat16)
+    vwin = torch.zeros_like(kwin)
+    q_out = torch.empty(B, Hq, D, device="cuda", dtype=torch.bfloat16)
+    call = ops.RopeAppendCall(qkv, cos, sin, pos, q_out, kwin, vwin, row)
+    for step in range(3):
+        qkv.copy_(torch.randn_like(qkv))
+        call.run()
+        v5 = qkv.view(B, 1, Hkv, 2 + G, D)
+        q = v5[..., :G, :].reshape(B, 1, Hq, D).transpose(1, 2)
+        qr, kr = pi.apply_rotary_pos_emb(q, v5[..., -2, :].transpose(1, 2), cos, sin, pos)
+        assert torch.equal(q_out, qr[:, :, 0]) and torch.equal(kwin[:, :, step], kr[:, :, 0])
+        assert torch.equal(vwin[:, :, step], v5[:, 0, :, -1, :])
+        pos.add_(1)
+        row.add_(1)
+    assert not kwin[:, :, 3:].any()

@@ -81,3 +81,45 @@ def test_decode_attn_token_values_split_path(bits):
         torch.cuda.synchronize()
         err = np.abs(to_np(out) - want)
         assert err.max() < MAX_ABS and err.mean() < MEAN_ABS, (splits, err.max(), err.mean())
+
+
+@pytest.mark.parametrize("bits", [1, 2])
+def test_token_quantiser_full_size_matches_the_torch_device_op_chain(bits):
+    """BASELINE layer shape (64 x 3328 x 8 x 128, bf16): the kernel's words / scales / minima equal what
+    the reference's sequence of torch ops (qjl/new_pack.py:64-72) gives on this GPU, and the words
+    unpack to codes in range that reach 0 and L in every group."""
+    from calibquant_amd import ops
+    B, T, H, D, L = 64, 3328, 8, 128, 2 ** bits - 1
+    torch.manual_seed(3)
+    x = torch.randn(B, T, H, D, device="cuda").to(torch.bfloat16)
+    words, scale, mins = ops.quantize_pack_token(x, bits)
+    g = x.permute(0, 2, 1, 3).reshape(B * H * T, D // 32, 32)
+    mn = g.amin(-1)
+    sc = (g.amax(-1) - mn) / L
+    data = g - mn.unsqueeze(-1)
+    data.div_(sc.unsqueeze(-1))
+    code = data.clamp_(0, L).round_().to(torch.int32)
+    assert torch.equal(scale.reshape(-1, 4), sc) and torch.equal(mins.reshape(-1, 4), mn)
+    shifts = torch.arange(0, 32, bits, device="cuda", dtype=torch.int64)
+    got = (words.reshape(-1, 4, bits, 1).to(torch.int64) & 0xFFFFFFFF) >> shifts & L      # (rows, groups, words, codes/word)
+    assert torch.equal(got.reshape(-1, 4, 32).to(torch.int32), code)
+    assert (code.amin(-1) == 0).all() and (code.amax(-1) == L).all()
+
+
+def test_decode_attn_token_values_full_batch_rows_are_independent():
+    """Batch 64 at the layer shape: rows fed identical inputs give identical outputs, and two rows
+    agree with the oracle."""
+    from calibquant_amd import ops
+    B, Hq, Hkv, T, R = 64, 32, 8, 3328, 128
+    c = _token_case(2, Hq, Hkv, T, R, 1, "bf16", seed=91)
+    g = case_to_gpu(c, "bf16")
+    rep = lambda t: t.repeat(B // 2, *([1] * (t.dim() - 1)))   # noqa: E731  rows 0,1,0,1,...
+    out = ops.decode_attn(rep(g["q"]), rep(g["ck"]), rep(g["cv"]), rep(g["sk"]), rep(g["zk"]), rep(g["sv"]),
+                          rep(g["zv"]), rep(g["kr"]), rep(g["vr"]), bits=1, v_mode="token")
+    torch.cuda.synchronize()
+    assert torch.equal(out[0::2], out[0:1].expand(B // 2, -1, -1))
+    assert torch.equal(out[1::2], out[1:2].expand(B // 2, -1, -1))
+    want = O.decode_attention(c["q"], c["ck"], c["cv"], c["sk"], c["zk"], c["sv"], c["zv"], c["kr"], c["vr"], 0, 1,
+                              v_token_group=32)
+    err = np.abs(to_np(out[:2]) - want)
+    assert err.max() < MAX_ABS and err.mean() < MEAN_ABS

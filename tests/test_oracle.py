@@ -311,3 +311,47 @@ def test_kivi_pack_little_endian_and_pv(bits):
     p = rng.random((1, 2, 9)).astype(np.float32)
     out = O.kivi_pv(p, words, s, mn, 32, bits)
     assert np.allclose(out, np.einsum("bht,bhtd->bhd", p, deq), atol=1e-5)
+
+
+def test_kivi_one_bit_words_are_packbits_little():
+    """1-bit per-token codes: the int32 words equal numpy's little-bit-order packing of the codes
+    (library routine), and every group's codes are the comparison with the group midpoint."""
+    rng = np.random.default_rng(5)
+    v = O.round_to(rng.standard_normal((2, 1, 7, 128)), "bf16")
+    words, s, mn = O.kivi_quantize_pack(v, 32, 1, "bf16")
+    codes = O.kivi_unpack(words, 1)
+    packed = np.packbits(codes.astype(np.uint8), axis=-1, bitorder="little")
+    assert np.array_equal(packed.reshape(2, 1, 7, 4, 4).view(np.uint32)[..., 0].view(np.int32), words)
+    g = v.reshape(2, 1, 7, 4, 32)
+    assert np.array_equal(mn, g.min(-1)) and np.array_equal(s, O.round_to(g.max(-1) - g.min(-1), "bf16"))
+    # away from the midpoint the code is just "above the middle of the group's range"
+    mid = (g.max(-1, keepdims=True) + g.min(-1, keepdims=True)) / 2
+    clear = np.abs(g - mid) > 0.02 * (g.max(-1, keepdims=True) - g.min(-1, keepdims=True))
+    assert np.array_equal(codes.reshape(g.shape)[clear], (g > mid)[clear].astype(np.int64))
+
+
+def test_decode_attention_per_token_values_brute_force():
+    """The per-token value branch of the oracle against python loops on explicitly dequantised
+    values scale*code + minimum (quantization.cu:116-117)."""
+    q, ck, _cv, sk, zk, _sv, _zv, kr, vr = _case(B=1, Hq=2, Hkv=1, D=32, T=6, R=2, bits=2, dtype="fp16", seed=11)
+    rng = np.random.default_rng(12)
+    v = O.round_to(rng.standard_normal((1, 1, 6, 32)), "fp16")
+    words, s, mn = O.kivi_quantize_pack(v, 32, 2, "fp16")
+    out = O.decode_attention(q, ck, words, sk, zk, s, mn, kr, vr, 1, 2, ftype=np.float64, v_token_group=32)
+    codes = O.kivi_unpack(words, 2)
+    ukc = O.unpack(ck, 2)
+    for h in range(2):
+        wi = [sum(float(q[0, h, d]) * float(sk[0, 0, d]) * (int(ukc[0, 0, t, d]) - float(zk[0, 0, d])) for d in range(32))
+              / math.sqrt(32) for t in range(6)]
+        mx, mi = max(wi), min(wi)
+        wi = [(w - mi) / (mx - mi + 1e-8) * ((mx - 3) - mi) + mi for w in wi]
+        wr = [sum(float(q[0, h, d]) * float(kr[0, 0, r, d]) for d in range(32)) / math.sqrt(32) for r in range(2)]
+        logits = wr[:1] + wi + wr[1:]
+        m = max(logits)
+        e = [math.exp(l - m) for l in logits]
+        p = [x / sum(e) for x in e]
+        for d in range(32):
+            vals = [float(vr[0, 0, 0, d])]
+            vals += [float(s[0, 0, t, 0]) * int(codes[0, 0, t, d]) + float(mn[0, 0, t, 0]) for t in range(6)]
+            vals += [float(vr[0, 0, 1, d])]
+            assert abs(out[0, h, d] - sum(pp * vv for pp, vv in zip(p, vals))) < 1e-9
