@@ -282,10 +282,9 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
         s_raw = sp[d];
         z_raw = zp[d];
     }
-    const uint4* ckp = has_img ? reinterpret_cast<const uint4*>(g.ck + (bh * g.T + t0) * NB)
-                               : static_cast<const uint4*>(g.q);
-    const uint4* cvp = has_img ? reinterpret_cast<const uint4*>(g.cv + (bh * g.T + t0) * NB)
-                               : static_cast<const uint4*>(g.q);
+    const int64_t code_off = has_img ? (bh * g.T + t0) * NB : 0;   // one offset for both code streams
+    const uint4* ckp = reinterpret_cast<const uint4*>((has_img ? g.ck : static_cast<const uint8_t*>(g.q)) + code_off);
+    const uint4* cvp = reinterpret_cast<const uint4*>((has_img ? g.cv : static_cast<const uint8_t*>(g.q)) + code_off);
     const U4* cvp4 = reinterpret_cast<const U4*>(cvp);
     const int last_u = has_img ? n * NB / 16 - 1 : 0;   // last valid 16-byte unit of either stream
     // residual tile: K slice (row = tid/8, 16 elements) and V slices (two rows, 8 elements)
@@ -293,10 +292,9 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
     // residual V: lane = (8-element slice ds, row slot): the slot's two low bits sit in the
     // two low lane bits so the final fold over slots is a quad permute
     const int ds = (tid >> 2) & 15, rslot = (tid & 3) | ((tid >> 6) << 2);
-    const uint16_t* kb = do_res ? static_cast<const uint16_t*>(g.kres) + b * g.rs_b + hkv * g.rs_h
-                                : static_cast<const uint16_t*>(g.q);
-    const uint16_t* vbp = do_res ? static_cast<const uint16_t*>(g.vres) + b * g.rs_b + hkv * g.rs_h
-                                 : static_cast<const uint16_t*>(g.q);
+    const int64_t res_off = do_res ? b * g.rs_b + hkv * g.rs_h : 0;   // one offset for both windows
+    const uint16_t* kb = static_cast<const uint16_t*>(do_res ? g.kres : g.q) + res_off;
+    const uint16_t* vbp = static_cast<const uint16_t*>(do_res ? g.vres : g.q) + res_off;
     const int last_r = do_res ? R - 1 : 0;
     const int64_t rs_r = do_res ? g.rs_r : 0;
     uint4 rk[2], rv[2];
@@ -330,11 +328,11 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
             const float zsum = (cpb0 == 8) ? oct_reduce(qs * z, OpSum(), 0.f) : quad_reduce(qs * z, OpSum(), 0.f);
             if (d % cpb0 == 0) qsz[(d / cpb0) * HPB + h] = zsum;
             if constexpr (BITS == 1) {
-                wbit[((d >> 3) * 8 + (7 - (d & 7))) * HPB + h] = qs;
+                wbit[((7 - (d & 7)) * NB + (d >> 3)) * HPB + h] = qs;   // [bit][byte position][head]
             } else {
                 const int sh = 6 - 2 * (d & 3);
-                wbit[((d >> 2) * 8 + sh) * HPB + h] = qs;
-                wbit[((d >> 2) * 8 + sh + 1) * HPB + h] = 2.0f * qs;
+                wbit[(sh * NB + (d >> 2)) * HPB + h] = qs;
+                wbit[((sh + 1) * NB + (d >> 2)) * HPB + h] = 2.0f * qs;
             }
         }
     }
@@ -377,14 +375,15 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
         V* ktab = reinterpret_cast<V*>(regA);           // [byte value][byte position]
         for (int e = tid; e < NB * 32; e += kNT) {
             const int j = e % NB, half = (e / NB) >> 4, v = (e / NB) & 15;
-            const V* wb = reinterpret_cast<const V*>(wbit) + j * 8 + half * 4;
+            // position-fastest: the lanes of a wave read consecutive entries
+            const V* wb = reinterpret_cast<const V*>(wbit) + half * 4 * NB + j;
             V acc;
             const V zs = reinterpret_cast<const V*>(qsz)[j];
 #pragma unroll
             for (int h = 0; h < HPB; ++h) acc.v[h] = half ? -zs.v[h] : 0.f;
 #pragma unroll
             for (int bt = 0; bt < 4; ++bt) {
-                const V w4 = wb[bt];
+                const V w4 = wb[bt * NB];
                 const float f = static_cast<float>((v >> bt) & 1);
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) acc.v[h] += f * w4.v[h];
@@ -672,6 +671,7 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
             // lane = (byte column j, slice c of its 8 bit lanes); a wave pass covers TPW tokens
             unsigned char* wtab = regA + wv * (L::NGRP * L::GPW * 16 * L::ESZH);   // [channel group][token group][16]
             const int j = lane / L::GPW, cs = lane % L::GPW;
+            const int wvu = __builtin_amdgcn_readfirstlane(wv);
             const int bg = lane >> 4, be = lane & 15;   // table build: group, entry
             f16x2_t bsel[4];
 #pragma unroll
@@ -719,7 +719,7 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                     }
                     __syncthreads();
                 }
-                for (int u = wv; u * L::TPW < vn; u += kNW) {
+                for (int u = wvu; u * L::TPW < vn; u += kNW) {   // wave-uniform loop control
                     const int tl = u * L::TPW;        // token offset inside the block
                     if (bg < L::GPW) {
                         // entry `be` of group `bg`: fp16 sum of the e values its bits select
