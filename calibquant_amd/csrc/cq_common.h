@@ -163,6 +163,27 @@ template <typename Op> __device__ __forceinline__ float wave_reduce(float v, Op 
     v = op(v, dpp_move<0x143, 0xc>(v, id));
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
+// The same over N values side by side: the chains are independent, so the cross-lane moves
+// of one fill the wait states of the others.
+template <int CTRL, int ROW_MASK, int N, typename Op>
+__device__ __forceinline__ void reduce_step(float* v, Op op, float id) {
+    float t[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) t[i] = dpp_move<CTRL, ROW_MASK>(v[i], id);
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] = op(v[i], t[i]);
+}
+template <int N, typename Op>
+__device__ __forceinline__ void wave_reduce_n(float* v, Op op, float id) {
+    reduce_step<0xB1, 0xf, N>(v, op, id);
+    reduce_step<0x4E, 0xf, N>(v, op, id);
+    reduce_step<0x141, 0xf, N>(v, op, id);
+    reduce_step<0x140, 0xf, N>(v, op, id);
+    reduce_step<0x142, 0xa, N>(v, op, id);
+    reduce_step<0x143, 0xc, N>(v, op, id);
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v[i]), 63));
+}
 __device__ __forceinline__ float wave_max(float v) { return key_float(wave_max_key(float_key(v))); }
 __device__ __forceinline__ float wave_min(float v) { return wave_reduce(v, OpMin(), INFINITY); }
 __device__ __forceinline__ float wave_sum(float v) { return wave_reduce(v, OpSum(), 0.0f); }

@@ -104,7 +104,7 @@ template <int BITS, int HPB, bool VTOK = false> struct Lay {
     static constexpr int SLOT = VTOK ? 16 : ESZ;    // bytes per token slot: logits, later e (+ 4 group scales)
     static constexpr int NGRP = VTOK ? kD / 32 : 1; // channel groups with tables of their own
     static constexpr int WTAB = kNW * NGRP * GPW * 16 * ESZH;
-    static constexpr int RW = cmax(2 * HPB, VTOK ? (NGRP + 1) * HPB : 0);   // widest set of per-wave partials
+    static constexpr int RW = cmax(3 * HPB, VTOK ? (NGRP + 1) * HPB : 0);   // per-wave partials: min/max + masked max, or the closing sums
     static constexpr int VSUB = kNT * kPF / BITS;   // V tokens staged at a time
     static constexpr int KR = kPF / BITS;           // K token rounds in flight per thread
     static constexpr int RED = kNW * PC * ESZ;
@@ -134,45 +134,52 @@ template <int BITS, int HPB, bool VTOK = false> struct Lay {
     }
 };
 
-// Block-wide reduction of HPB values with `op`; result broadcast to all threads
-// (wave-uniform, so it can live in scalar registers).
-template <int HPB, typename Op>
-__device__ __forceinline__ void block_reduce(float* v, float* red, Op op, float identity) {
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+// One exchange step of an integer-key maximum, N values side by side: the N chains are
+// independent, so the cross-lane moves of one fill the wait states of the others.
+template <int N, int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ void max_step(int* k) {
+    constexpr int lo = static_cast<int>(0x80000000u);
+    int t[N];
 #pragma unroll
-    for (int h = 0; h < HPB; ++h) {
-        const float x = wave_reduce(v[h], op, identity);
-        if (lane == 0) red[w * HPB + h] = x;
-    }
-    __syncthreads();
-    static_assert(kNW <= 16, "second stage folds at most 16 wave partials");
+    for (int h = 0; h < N; ++h) t[h] = dpp_move_i<CTRL, ROW_MASK>(k[h], lo);
 #pragma unroll
-    for (int h = 0; h < HPB; ++h) {
-        float x = (lane < kNW) ? red[lane * HPB + h] : identity;
-        x = row_reduce(x, op, identity);   // lanes 0..15 hold the partials
-        v[h] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, x)));
-    }
-    __syncthreads();
+    for (int h = 0; h < N; ++h) k[h] = max(k[h], t[h]);
 }
 
 // Block-wide maximum of N values (integer keys, see float_key); result wave-uniform.
+// One barrier; `red` (kNW * N words) must not be rewritten before the next barrier of the caller.
 template <int N>
 __device__ __forceinline__ void block_max(float* v, float* red) {
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     int* redi = reinterpret_cast<int*>(red);
+    int k[N];
 #pragma unroll
-    for (int h = 0; h < N; ++h) {
-        const int x = wave_max_key(float_key(v[h]));
-        if (lane == 0) redi[w * N + h] = x;
+    for (int h = 0; h < N; ++h) k[h] = float_key(v[h]);
+    max_step<N, 0xB1>(k);
+    max_step<N, 0x4E>(k);
+    max_step<N, 0x141>(k);
+    max_step<N, 0x140>(k);
+    max_step<N, 0x142, 0xa>(k);
+    max_step<N, 0x143, 0xc>(k);
+    if (lane == 63) {   // the last lane holds the wave's maxima
+#pragma unroll
+        for (int h = 0; h < N; ++h) redi[w * N + h] = k[h];
     }
     __syncthreads();
+    static_assert(kNW <= 16, "second stage folds at most 16 wave partials");
+    int x[N];
 #pragma unroll
-    for (int h = 0; h < N; ++h) {
-        int x = (lane < kNW) ? redi[lane * N + h] : static_cast<int>(0x80000000u);
-        x = row_max_key(x);
-        v[h] = key_float(__builtin_amdgcn_readfirstlane(x));
+    for (int h = 0; h < N; ++h) x[h] = static_cast<int>(0x80000000u);
+    if (lane < kNW) {
+#pragma unroll
+        for (int h = 0; h < N; ++h) x[h] = redi[lane * N + h];
     }
-    __syncthreads();
+    max_step<N, 0xB1>(x);   // lanes 0..15 hold the partials
+    max_step<N, 0x4E>(x);
+    max_step<N, 0x141>(x);
+    max_step<N, 0x140>(x);
+#pragma unroll
+    for (int h = 0; h < N; ++h) v[h] = key_float(__builtin_amdgcn_readfirstlane(x[h]));
 }
 
 // Unit decomposition of a 1-D grid.  Consecutive work ids share packed codes
@@ -536,7 +543,7 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
 
         if (n > 0) {
             // The K table is dead: stage the first block of packed V rows in its place
-            // (ordered by the barriers of block_reduce).  Layout: [unit of TPW tokens]
+            // (ordered by the barrier of block_max).  Layout: [unit of TPW tokens]
             // [byte column][token], so the 4 bytes that the 4 tokens of a group have in one
             // column form one dword.  A quad of lanes holds a group (tokens are
             // lane-consecutive): per dword of its 16-byte piece the quad transposes a 4 x 4 byte
@@ -608,7 +615,7 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                     }
                     *reinterpret_cast<V*>(slot(tt)) = w;
                 }
-                block_max<HPB>(lm, red);
+                block_max<HPB>(lm, red + kNW * 2 * HPB);   // the first reduction's words may still be read
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) { m_img[h] = lm[h]; slope[h] = 1.0f; tmin[h] = 0.f; mn[h] = 0.f; }
             } else {
@@ -800,26 +807,28 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
             load_res_v(0, rv);
             // per-wave partial sums of e (and of e * minimum), folded by the output threads below
             constexpr int kSums = VTOK ? (L::NGRP + 1) * HPB : HPB;
-#pragma unroll
-            for (int h = 0; h < HPB; ++h) {
-                const float x = wave_sum(ls[h]);
-                if (lane == 0) red[wv * kSums + h] = x;
-            }
+            wave_reduce_n<HPB>(ls, OpSum(), 0.f);
             if constexpr (VTOK) {
 #pragma unroll
-                for (int i = 0; i < L::NGRP * HPB; ++i) {
-                    const float x = wave_sum(cma[i]);
-                    if (lane == 0) red[wv * kSums + HPB + i] = x;
+                for (int gi = 0; gi < L::NGRP; ++gi) wave_reduce_n<HPB>(cma + gi * HPB, OpSum(), 0.f);
+            }
+            if (lane == 0) {
+#pragma unroll
+                for (int h = 0; h < HPB; ++h) red[wv * kSums + h] = ls[h];
+                if constexpr (VTOK) {
+#pragma unroll
+                    for (int i = 0; i < L::NGRP * HPB; ++i) red[wv * kSums + HPB + i] = cma[i];
                 }
             }
             __syncthreads();
-            V* redv = reinterpret_cast<V*>(regA);  // [wave][PC]
+            // head-major, so that the fold below reads consecutive words with consecutive lanes
+            float* redv = reinterpret_cast<float*>(regA);  // [wave][head][bit lane]
 #pragma unroll
-            for (int m = 0; m < L::MPL; ++m) {
-                V a4;
+            for (int h = 0; h < HPB; ++h) {
+                Vec<L::MPL> a4;
 #pragma unroll
-                for (int h = 0; h < HPB; ++h) a4.v[h] = acc[m][h];
-                redv[wv * L::PC + j * 8 + cs * L::MPL + m] = a4;
+                for (int m = 0; m < L::MPL; ++m) a4.v[m] = acc[m][h];
+                *reinterpret_cast<Vec<L::MPL>*>(redv + (wv * HPB + h) * L::PC + j * 8 + cs * L::MPL) = a4;
             }
             __syncthreads();
             if (tid < HPB * kD) {
@@ -832,11 +841,11 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                 const int lane_hi = VTOK ? cb + 8 - BITS * (c + 1) : cb + BITS * c;   // bit lane of the code's top bit
                 if constexpr (BITS == 1) {
 #pragma unroll
-                    for (int w = 0; w < kNW; ++w) a += redv[w * L::PC + lane_hi].v[h];
+                    for (int w = 0; w < kNW; ++w) a += redv[(w * HPB + h) * L::PC + lane_hi];
                 } else {
 #pragma unroll
                     for (int w = 0; w < kNW; ++w)
-                        a += 2.0f * redv[w * L::PC + lane_hi].v[h] + redv[w * L::PC + lane_hi + 1].v[h];
+                        a += 2.0f * redv[(w * HPB + h) * L::PC + lane_hi] + redv[(w * HPB + h) * L::PC + lane_hi + 1];
                 }
                 float lh = 0.f;   // sum of e of this thread's head
 #pragma unroll
@@ -944,18 +953,18 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) accv[k][h] = quad_reduce(accv[k][h], OpSum(), 0.f);
             __syncthreads();
-            float* red2 = reinterpret_cast<float*>(regA);  // [wave][kD][HPB]
+            float* red2 = reinterpret_cast<float*>(regA);  // [wave][head][kD]: the fold reads consecutive words
             if ((lane & 3) == 0) {
 #pragma unroll
                 for (int k = 0; k < 8; ++k)
 #pragma unroll
-                    for (int h = 0; h < HPB; ++h) red2[(wv * kD + ds * 8 + k) * HPB + h] = accv[k][h];
+                    for (int h = 0; h < HPB; ++h) red2[(wv * HPB + h) * kD + ds * 8 + k] = accv[k][h];
             }
             __syncthreads();
             if (tid < HPB * kD) {
                 const int h = tid / kD, d = tid % kD;
 #pragma unroll
-                for (int w = 0; w < kNW; ++w) o_res += red2[(w * kD + d) * HPB + h];
+                for (int w = 0; w < kNW; ++w) o_res += red2[(w * HPB + h) * kD + d];
             }
         }
 
