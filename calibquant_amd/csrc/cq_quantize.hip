@@ -111,20 +111,33 @@ __device__ __forceinline__ float key_value(int key) {   // key >= 0: pattern key
 }
 
 // ---- 2. statistics ---------------------------------------------------------
-// grid (B*H), D threads.  The op chain of calibquant.py:27-34 with one
-// rounding per op; `tensor / python_scalar` is a multiply by the fp32
-// reciprocal, as torch's device kernel does.
+// grid (B*H), 1024 threads = 1024/D parts x D channels: thread (p, d) folds every (1024/D)-th chunk
+// partial of channel d; after the fold, part 0 writes the statistics and parts 1..3 search one
+// threshold each.
+// The op chain of calibquant.py:27-34 with one rounding per op; `tensor / python_scalar` is
+// a multiply by the fp32 reciprocal, as torch's device kernel does.
+constexpr int kStatThreads = 1024;
 template <typename DT>
 __global__ void stats_kernel(const float* __restrict__ part, QuantGeom g, float clip, float levels,
                              uint16_t* __restrict__ scale, uint16_t* __restrict__ zero, float* __restrict__ thr) {
     const int bh = blockIdx.x;
-    const int d = threadIdx.x;
-    if (d >= g.D) return;
+    const int d = threadIdx.x % g.D;
+    const int pt = threadIdx.x / g.D;
+    const int nparts = kStatThreads / g.D;   // >= 4 for D <= 256
+    __shared__ float sh[2 * kStatThreads];   // [part][2][D]
     float a = INFINITY, z = -INFINITY;
     const float* p = part + static_cast<int64_t>(bh) * g.nchunk * 2 * g.D;
-    for (int c = 0; c < g.nchunk; ++c) {
+#pragma unroll 4
+    for (int c = pt; c < g.nchunk; c += nparts) {   // independent loads: four pairs in flight
         a = fminf(a, p[c * 2 * g.D + d]);
         z = fmaxf(z, p[c * 2 * g.D + g.D + d]);
+    }
+    sh[(pt * 2) * g.D + d] = a;
+    sh[(pt * 2 + 1) * g.D + d] = z;
+    __syncthreads();
+    for (int q = 0; q < nparts; ++q) {
+        a = fminf(a, sh[(q * 2) * g.D + d]);
+        z = fmaxf(z, sh[(q * 2 + 1) * g.D + d]);
     }
     const float x_min = rnd<DT>(a * clip);
     const float x_max = rnd<DT>(z * clip);
@@ -132,36 +145,38 @@ __global__ void stats_kernel(const float* __restrict__ part, QuantGeom g, float 
     const float inv_levels = __fdiv_rn(1.0f, levels);
     const float s = rnd<DT>(diff * inv_levels);
     const float zp = rnd<DT>(__fdiv_rn(-x_min, s));
-    scale[static_cast<int64_t>(bh) * g.D + d] = static_cast<uint16_t>(Cvt<DT>::from_float(s));
-    zero[static_cast<int64_t>(bh) * g.D + d] = static_cast<uint16_t>(Cvt<DT>::from_float(zp));
-
     // thresholds thr[k-1] = smallest storage value whose code is >= k (k = 1..L), kept as
     // [k][channel].  NaN in thr[0]: the step-function argument does not hold for this channel
     // (scale not positive and finite, or zero-point NaN) and emit evaluates the chain itself.
     float* o = thr + static_cast<int64_t>(bh) * 3 * g.D + d;
     const bool monotone = s > 0.0f && s < INFINITY && zp == zp;
-    const int nlev = static_cast<int>(levels);
-    for (int k = 1; k <= 3; ++k) {
-        float t = NAN;   // no value reaches code k
-        if (monotone && k <= nlev) {
-            int lo = Keys<DT>::lo, hi = Keys<DT>::hi;   // invariant: code(lo) < k (or lo is the floor), answer in (lo, hi]
-            if (quant_value<DT>(key_value<DT>(hi), s, zp, levels) >= static_cast<float>(k)) {
-                if (quant_value<DT>(key_value<DT>(lo), s, zp, levels) >= static_cast<float>(k)) {
-                    hi = lo;
-                } else {
-                    while (hi - lo > 1) {
-                        const int mid = lo + (hi - lo) / 2;
-                        if (quant_value<DT>(key_value<DT>(mid), s, zp, levels) >= static_cast<float>(k)) hi = mid;
-                        else lo = mid;
-                    }
-                }
-                t = key_value<DT>(hi);
-            }
-        }
-        if (k == 1 && !monotone) t = NAN;
-        o[(k - 1) * g.D] = t;
+    if (pt == 0) {
+        scale[static_cast<int64_t>(bh) * g.D + d] = static_cast<uint16_t>(Cvt<DT>::from_float(s));
+        zero[static_cast<int64_t>(bh) * g.D + d] = static_cast<uint16_t>(Cvt<DT>::from_float(zp));
+        return;
     }
-    if (!monotone) o[g.D] = 1.0f;   // thr[1] distinguishes "not monotone" (non-NaN) from "code 1 unreachable" (NaN)
+    if (pt > 3) return;
+    const int nlev = static_cast<int>(levels);
+    const int k = pt;   // this thread's level
+    float t = NAN;      // no value reaches code k
+    if (monotone && k <= nlev) {
+        int lo = Keys<DT>::lo, hi = Keys<DT>::hi;   // invariant: code(lo) < k (or lo is the floor), answer in (lo, hi]
+        if (quant_value<DT>(key_value<DT>(hi), s, zp, levels) >= static_cast<float>(k)) {
+            if (quant_value<DT>(key_value<DT>(lo), s, zp, levels) >= static_cast<float>(k)) {
+                hi = lo;
+            } else {
+                while (hi - lo > 1) {
+                    const int mid = lo + (hi - lo) / 2;
+                    if (quant_value<DT>(key_value<DT>(mid), s, zp, levels) >= static_cast<float>(k)) hi = mid;
+                    else lo = mid;
+                }
+            }
+            t = key_value<DT>(hi);
+        }
+    }
+    // thr[1] distinguishes "not monotone" (non-NaN) from "code 1 unreachable" (NaN)
+    if (!monotone) t = (k == 2) ? 1.0f : NAN;
+    o[(k - 1) * g.D] = t;
 }
 
 // ---- 3. emit -----------------------------------------------------------------
@@ -420,7 +435,7 @@ static int run_quant(const void* x, QuantGeom g, int bits, float clip, uint8_t* 
     CQ_LAUNCH_CHECK();
     const float levels = static_cast<float>((1 << bits) - 1);
     float* thr = ws + static_cast<size_t>(g.B) * g.H * g.nchunk * 2 * g.D;
-    hipLaunchKernelGGL(stats_kernel<DT>, dim3(g.B * g.H), dim3(g.D), 0, st, ws, g, clip, levels, sp, zp, thr);
+    hipLaunchKernelGGL(stats_kernel<DT>, dim3(g.B * g.H), dim3(kStatThreads), 0, st, ws, g, clip, levels, sp, zp, thr);
     CQ_LAUNCH_CHECK();
     uint16_t* xqp = static_cast<uint16_t*>(xq);
     if (xq) {
