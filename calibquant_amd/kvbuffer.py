@@ -23,6 +23,23 @@ class GrowingKV:
                 and past[0].shape[2] == self.len and past[0].shape[:2] == self.k.shape[:2]
                 and past[0].stride() == self.k.stride())
 
+    def reserve(self, past: Optional[Tuple[torch.Tensor, torch.Tensor]], need: int, like: torch.Tensor,
+                shape_bh: Tuple[int, int], D: int) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Make the buffers hold `past` (None, or a (B, H, R, D) pair) with room for `need` rows in
+        all, and return the whole buffers (B, H, capacity, D); rows beyond R are for the caller to fill."""
+        R = 0 if past is None else past[0].shape[2]
+        if not self._owns(past) or need > self.k.shape[2]:
+            B, H = shape_bh
+            cap = need + max(256, need // 8)
+            k = torch.empty((B, H, cap, D), dtype=like.dtype, device=like.device)
+            v = torch.empty_like(k)
+            if R:
+                k[:, :, :R] = past[0]
+                v[:, :, :R] = past[1]
+            self.k, self.v = k, v
+            self.len = R
+        return self.k, self.v
+
     def append(self, past: Optional[Tuple[torch.Tensor, torch.Tensor]], k_new: torch.Tensor,
                v_new: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
         """past: None or the (K, V) pair returned earlier (or any (B, H, R, D) pair);
@@ -30,15 +47,13 @@ class GrowingKV:
         B, H, n, D = k_new.shape
         R = 0 if past is None else past[0].shape[2]
         need = R + n
-        if not self._owns(past) or need > self.k.shape[2]:
-            cap = need + max(256, need // 8)
-            k = torch.empty((B, H, cap, D), dtype=k_new.dtype, device=k_new.device)
-            v = torch.empty_like(k)
-            if R:
-                k[:, :, :R] = past[0]
-                v[:, :, :R] = past[1]
-            self.k, self.v = k, v
+        self.reserve(past, need, k_new, (B, H), D)
         self.k[:, :, R:need] = k_new
         self.v[:, :, R:need] = v_new
+        self.len = need
+        return self.k[:, :, :need], self.v[:, :, :need]
+
+    def extended(self, need: int) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Views of the first `need` rows after the caller filled rows [len, need) in place."""
         self.len = need
         return self.k[:, :, :need], self.v[:, :, :need]

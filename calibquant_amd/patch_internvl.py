@@ -140,6 +140,10 @@ def forward_internlm2_calibquant(self, hidden_states: torch.Tensor, attention_ma
 
     # (h gs d) de-interleave of the fused projection: views only (patch_internvl.py:214-234)
     qkv = self.wqkv(hidden_states).view(bsz, q_len, Hkv, 2 + G, D)
+    if (q_len == 1 and past_key_value is not None and position_ids is not None and position_ids.is_cuda
+            and position_ids.dtype == torch.int64 and position_ids.numel() == bsz and qkv.is_contiguous()
+            and qkv.dtype in (torch.bfloat16, torch.float16)):
+        return _decode_step_fused(self, qkv, position_ids, past_key_value, attention_mask, use_cache)
     query_states = qkv[..., :G, :].reshape(bsz, q_len, Hq, D).transpose(1, 2)     # (B, Hq, q, D)
     key_states = qkv[..., -2, :].transpose(1, 2)                                   # (B, Hkv, q, D)
     value_states = qkv[..., -1, :].transpose(1, 2)
@@ -233,6 +237,64 @@ def forward_internlm2_calibquant(self, hidden_states: torch.Tensor, attention_ma
         self._cq_call = call if mask is None else None
     attn_output = self.wo(out.reshape(bsz, 1, self.hidden_size))
     return attn_output, None, past_key_value
+
+
+def _decode_step_fused(self, qkv, position_ids, past_key_value, attention_mask, use_cache):
+    """One decode step with the split of the fused projection, the rotary embedding of q and k and
+    the append of the new key / value row in one launch (`cq_rope_append`, bit-identical to the
+    chain of torch ops of patch_internvl.py:119-138, 219-266), then the fused attention launch."""
+    bsz = qkv.shape[0]
+    G, D, Hq = self.num_key_value_groups, self.head_dim, self.num_heads
+    Hkv = Hq // G
+    S, T = self.sprompt_len, self.image_token_num
+    R0 = past_key_value[0].shape[2]
+    R = R0 + 1
+    kv_seq_len = R + T
+    # rotary tables in the storage dtype, kept on the module with room to spare
+    tabs = getattr(self, "_cq_rope_tables", None)
+    if tabs is None or tabs[0].shape[0] < kv_seq_len or tabs[0].dtype != qkv.dtype or tabs[0].device != qkv.device:
+        cos, sin = self.rotary_emb(qkv, seq_len=kv_seq_len + 512)
+        tabs = self._cq_rope_tables = (cos.contiguous(), sin.contiguous())
+    if not hasattr(self, "_cq_window"):
+        self._cq_window = GrowingKV()
+    win = self._cq_window
+    k_buf, v_buf = win.reserve(past_key_value, R, qkv, (bsz, Hkv), D)
+    # a cell that holds the row index on the device: cell i of a ramp holds i
+    rows = getattr(self, "_cq_row_ramp", None)
+    if rows is None or rows.numel() <= R0 or rows.device != qkv.device:
+        rows = self._cq_row_ramp = torch.arange(max(4096, 2 * R), dtype=torch.int64, device=qkv.device)
+    row = rows[R0:R0 + 1]
+    q1 = torch.empty((bsz, Hq, D), dtype=qkv.dtype, device=qkv.device)
+    rope = getattr(self, "_cq_rope_call", None)
+    with torch.cuda.device(qkv.device):
+        if rope is None or rope._args[2:6] != (bsz, Hq, Hkv, D) or rope._keep[1] is not tabs[0]:
+            rope = self._cq_rope_call = ops.RopeAppendCall(qkv, tabs[0], tabs[1], position_ids, q1, k_buf, v_buf, row)
+            rope.run()
+        else:
+            rope.step(qkv, position_ids, q1, k_buf, v_buf, row)
+    k_res, v_res = win.extended(R)
+    past_key_value = (k_res, v_res) if use_cache else None
+    mask = None
+    if attention_mask is not None:
+        if attention_mask.size() != (bsz, 1, 1, kv_seq_len):
+            raise ValueError(f"Attention mask should be of size {(bsz, 1, 1, kv_seq_len)}, "
+                             f"but is {attention_mask.size()}")
+        mask = attention_mask[:, 0, 0, :]
+    call = getattr(self, "_cq_call", None)
+    if (mask is None and call is not None and call.args.B == bsz and call.workspace_bytes == 0
+            and call.args.dtype == (0 if q1.dtype == torch.bfloat16 else 1)):
+        out = call.step(q1, k_res, v_res, torch.empty_like(q1))
+    else:
+        stats = self._cq_stats if T > 0 else (None,) * 4
+        call = ops.DecodeCall(q1, self.encoded_features_k if T > 0 else None,
+                              self.encoded_features_v if T > 0 else None, stats[0], stats[1], stats[2], stats[3],
+                              k_res, v_res, sprompt_len=min(S, R), bits=self.bits_k, calibrate=self.normalize,
+                              calib_off_max=CALIB_OFFSET_MAX, calib_off_min=CALIB_OFFSET_MIN, mask=mask,
+                              v_mode=self.v_mode)
+        with torch.cuda.device(call.device):
+            out = call.run()
+        self._cq_call = call if mask is None else None
+    return self.wo(out.reshape(bsz, 1, self.hidden_size)), None, past_key_value
 
 
 def _no_qjl(*args, **kwargs):

@@ -65,6 +65,40 @@ def test_patched_forward_decode_matches_oracle_on_one_layer():
         assert err.max().item() < 2e-2 and err.mean().item() < 2e-3
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fused_decode_step_equals_the_unfused_op_chain(dtype):
+    """Several decode steps through the one-launch split + rotary + append path and through the
+    chain of torch ops (forced by int32 position ids): same outputs and same window, bit for bit."""
+    from calibquant_amd import patch_internvl as pi
+    from calibquant_amd.internlm2 import InternLM2Attention, InternLM2Config
+    cfg = InternLM2Config.tiny()
+    B, S, T, TXT = 3, 4, 130, 9
+    N = S + T + TXT
+    outs, wins = [], []
+    for fused in (True, False):
+        torch.manual_seed(7)
+        att = InternLM2Attention(cfg).cuda().to(dtype)
+        att.cq_sprompt_len, att.image_token_num = S, T
+        x = torch.randn(B, N, cfg.hidden_size, device="cuda", dtype=dtype)
+        pos = torch.arange(N, device="cuda")[None].expand(B, N)
+        with torch.no_grad():
+            _, _, past = pi.forward_internlm2_calibquant(att, x, None, pos, None, False, True)
+            step_out = []
+            for i in range(300):   # beyond the first window capacity: the buffers are regrown on the way
+                xd = torch.randn(B, 1, cfg.hidden_size, device="cuda", dtype=dtype)
+                posd = torch.full((B, 1), N + i, device="cuda", dtype=torch.long)
+                o, _, past = pi.forward_internlm2_calibquant(att, xd, None, posd if fused else posd.int(), past,
+                                                            False, True)
+                if i % 37 == 0 or i == 299:
+                    step_out.append(o.clone())
+        assert hasattr(att, "_cq_rope_call") == fused
+        outs.append(torch.stack(step_out))
+        wins.append((past[0].clone(), past[1].clone()))
+    assert wins[0][0].shape == (B, cfg.num_key_value_heads, S + TXT + 300, 128)
+    assert torch.equal(wins[0][0], wins[1][0]) and torch.equal(wins[0][1], wins[1][1])
+    assert torch.equal(outs[0], outs[1])
+
+
 def test_patched_model_without_image_tokens_equals_the_fp_model():
     """With zero packed tokens the quantised path is plain attention over the fp window."""
     from calibquant_amd import patch_internvl as pi
