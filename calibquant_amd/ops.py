@@ -292,22 +292,23 @@ class RopeAppendCall:
         if pos.dtype != torch.int64 or row.dtype != torch.int64 or pos.numel() != B or row.numel() != 1:
             raise _lib.CalibQuantError("rope_append: pos (B int64) / row (1 int64) expected")
         self._lib = _lib.load()
-        self._keep = (qkv, cos, sin, pos, q_out, k_win, v_win, row)
         self.device = qkv.device
-        self._args = (qkv.data_ptr(), dt, B, Hq, Hkv, D, cos.data_ptr(), sin.data_ptr(), cos.shape[0],
-                      pos.data_ptr(), pos.reshape(B).stride(0), q_out.data_ptr(), k_win.data_ptr(), v_win.data_ptr(),
-                      k_win.stride(0), k_win.stride(1), k_win.stride(2), cap, row.data_ptr())
+        self.geometry = (B, Hq, Hkv, D)          # what a prepared call can be re-aimed within
+        self.tables = (cos, sin)
+        self._fixed = (dt, B, Hq, Hkv, D, cos.data_ptr(), sin.data_ptr(), cos.shape[0])
+        self._aim(qkv, pos, q_out, k_win, v_win, row)
+
+    def _aim(self, qkv, pos, q_out, k_win, v_win, row) -> None:
+        self._keep = (qkv, pos, q_out, k_win, v_win, row)
+        self._args = (qkv.data_ptr(),) + self._fixed + (
+            pos.data_ptr(), pos.reshape(-1).stride(0), q_out.data_ptr(), k_win.data_ptr(), v_win.data_ptr(),
+            k_win.stride(0), k_win.stride(1), k_win.stride(2), k_win.shape[2], row.data_ptr())
 
     def step(self, qkv, pos, q_out, k_win, v_win, row) -> None:
         """Re-aim the prepared launch at this step's projection output, position ids, query
-        output, window buffers (same shape class, possibly regrown) and row cell, and launch.
+        output, window buffers (same geometry, possibly regrown) and row cell, and launch.
         Only pointers, strides and the capacity change; no validation beyond the C entry point's."""
-        a = list(self._args)
-        a[0], a[9], a[10], a[11] = qkv.data_ptr(), pos.data_ptr(), pos.reshape(-1).stride(0), q_out.data_ptr()
-        a[12], a[13] = k_win.data_ptr(), v_win.data_ptr()
-        a[14], a[15], a[16], a[17], a[18] = k_win.stride(0), k_win.stride(1), k_win.stride(2), k_win.shape[2], row.data_ptr()
-        self._args = tuple(a)
-        self._keep = (qkv, self._keep[1], self._keep[2], pos, q_out, k_win, v_win, row)
+        self._aim(qkv, pos, q_out, k_win, v_win, row)
         self.run()
 
     def run(self) -> None:

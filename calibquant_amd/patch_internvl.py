@@ -267,7 +267,7 @@ def _decode_step_fused(self, qkv, position_ids, past_key_value, attention_mask, 
     q1 = torch.empty((bsz, Hq, D), dtype=qkv.dtype, device=qkv.device)
     rope = getattr(self, "_cq_rope_call", None)
     with torch.cuda.device(qkv.device):
-        if rope is None or rope._args[2:6] != (bsz, Hq, Hkv, D) or rope._keep[1] is not tabs[0]:
+        if rope is None or rope.geometry != (bsz, Hq, Hkv, D) or rope.tables[0] is not tabs[0]:
             rope = self._cq_rope_call = ops.RopeAppendCall(qkv, tabs[0], tabs[1], position_ids, q1, k_buf, v_buf, row)
             rope.run()
         else:
