@@ -334,7 +334,7 @@ def main():
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py: this build measures one GPU only (asked for {a.gpus}); "
-              "the path shards over batch and kv-heads without exchange, see DESIGN.md", file=sys.stderr)
+              "the path shards over batch rows and kv-heads without any exchange between GPUs", file=sys.stderr)
         sys.exit(2)
 
     import torch
