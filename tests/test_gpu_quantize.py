@@ -54,6 +54,21 @@ def test_quantize_pack_reads_the_strided_wqkv_view(ops, dtype):
         assert np.array_equal(codes.cpu().numpy(), oc)
 
 
+@pytest.mark.parametrize("bits", [1, 2])
+def test_quantize_pack_long_context_single_sequence(ops, bits):
+    """One sequence of 32 768 tokens: few (batch, head) pairs, so the statistics of a channel are
+    folded from 256 chunk partials and every threshold level is searched by its own threads."""
+    B, T, H, D = 1, 32768, 2, 128
+    print(f"case quantize_pack long context bits={bits}", flush=True)
+    k, v = O.synth_kv(B, T, H, D, "bf16", seed=77)
+    for x, clip in zip((k, v), CLIPS[bits]):
+        codes, s, z = ops.quantize_pack(to_gpu(x, "bf16"), bits, clip)
+        torch.cuda.synchronize()
+        oc, os_, oz = O.quantize_pack(x, bits, clip, "bf16")
+        assert same_bits(to_np(s), os_) and same_bits(to_np(z), oz)
+        assert np.array_equal(codes.cpu().numpy(), oc)
+
+
 def test_quantize_pack_constant_channel_matches_ieee_reference(ops):
     x = np.random.default_rng(1).standard_normal((1, 64, 2, 128)).astype(np.float32)
     x = O.round_to(x, "bf16")
