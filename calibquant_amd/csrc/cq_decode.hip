@@ -33,6 +33,7 @@
 #include "cq_common.h"
 
 #include <atomic>
+#include <type_traits>
 
 namespace cq {
 
@@ -100,7 +101,14 @@ template <int BITS, int HPB, bool VTOK = false> struct Lay {
     static constexpr int ESZ = HPB * 4;             // bytes per fp32 table entry / logits slot
     static constexpr int HW = HPB >= 2 ? HPB / 2 : 1;   // 32-bit words per packed-fp16 entry
     static constexpr int ESZH = HW * 4;             // bytes per packed-fp16 table entry
-    static constexpr int KT = NB * 256 * ESZ;       // K table bytes
+    // The byte-indexed K table covers NBP byte positions at a time: all of them when that fits
+    // 64 KB, else half of them in each of two passes over the chunk's rows (one 16-byte piece
+    // of a 2-bit row per pass), the first pass's partial logits waiting in the token slots.
+    static constexpr int KPASS = (NB * 256 * ESZ > 64 * 1024) ? 2 : 1;
+    static constexpr int NBP = NB / KPASS;          // byte positions per pass
+    static constexpr int PPP = BITS / KPASS;        // 16-byte pieces of a row per pass
+    static constexpr int KT = NBP * 256 * ESZ;      // K table bytes
+    static_assert(KPASS == 1 || (KPASS == 2 && BITS == 2), "a pass consumes whole 16-byte pieces");
     static constexpr int SLOT = VTOK ? 16 : ESZ;    // bytes per token slot: logits, later e (+ 4 group scales)
     static constexpr int NGRP = VTOK ? kD / 32 : 1; // channel groups with tables of their own
     static constexpr int WTAB = kNW * NGRP * GPW * 16 * ESZH;
@@ -398,46 +406,39 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
             nib[e] = acc;
         }
         __syncthreads();
-        for (int e = tid; e < NB * 256; e += kNT) {
-            const int j = e % NB, v = e / NB;
-            const V hi = nib[(16 + (v >> 4)) * NB + j];
-            const V lo = nib[(v & 15) * NB + j];
-            V o;
-#pragma unroll
-            for (int h = 0; h < HPB; ++h) o.v[h] = hi.v[h] + lo.v[h];
-            ktab[e] = o;
-        }
-        __syncthreads();
 
         // ---- phase 3: logits of the chunk ------------------------------------------------
-        // Lane l walks the byte positions in the order k ^ (l mod NB): in every step the
-        // lanes that the LDS serves together read NB distinct positions of the
+        // Lane l walks the byte positions of a pass in the order k ^ (l mod NBP): in every step
+        // the lanes that the LDS serves together read NBP distinct positions of the
         // position-fastest table, i.e. distinct banks whatever the byte values are.  The
         // row is permuted by the same XOR once, so step k finds its byte at a fixed place.
-        // The NB terms are added as a balanced binary tree over k; an XOR of the leaf index
+        // The NBP terms are added as a balanced binary tree over k; an XOR of the leaf index
         // only swaps the two children of some tree levels, so every lane gets bit-identical
         // logits for identical rows.
-        constexpr int NW32 = NB / 4;
-        const int skew = lane % NB;
+        constexpr int NBP = L::NBP;
+        constexpr int NW32 = NBP / 4;
+        const int skew = lane % NBP;
         // byte i of a word <- byte i ^ (skew & 3)
         const uint32_t bsel = (0x03020100u ^ (0x01010101u * (skew & 3)));
-        uint32_t pofs[NB];   // byte offset of position k ^ skew inside a table row
+        uint32_t pofs[NBP];   // byte offset of position k ^ skew inside a table row
 #pragma unroll
-        for (int k = 0; k < NB; ++k) pofs[k] = (k ^ skew) * L::ESZ;
+        for (int k = 0; k < NBP; ++k) pofs[k] = (k ^ skew) * L::ESZ;
         const unsigned char* ktab_b = regA;
         // With 256-byte table rows the address of a look-up is two bytes side by side, the
         // byte value above the position offset: one byte permute builds it from the row word
         // and a word holding four position offsets.
-        constexpr bool kPermAddr = (NB * L::ESZ == 256);
-        uint32_t pofs4[NB / 4];
+        constexpr bool kPermAddr = (NBP * L::ESZ == 256);
+        uint32_t pofs4[NBP / 4];
 #pragma unroll
-        for (int i = 0; i < NB / 4; ++i)
+        for (int i = 0; i < NBP / 4; ++i)
             pofs4[i] = pofs[4 * i] | (pofs[4 * i + 1] << 8) | (pofs[4 * i + 2] << 16) | (pofs[4 * i + 3] << 24);
-        auto token_logits = [&](int tt, const uint4* c) {
+        // c: the L::PPP pieces of the row that pass P covers
+        auto token_logits = [&](auto pass_c, int tt, const uint4* c) {
+            constexpr int P = decltype(pass_c)::value;
             if (tt < n) {
                 uint32_t w[NW32];
 #pragma unroll
-                for (int i = 0; i < BITS; ++i) {
+                for (int i = 0; i < L::PPP; ++i) {
                     w[4 * i + 0] = c[i].x; w[4 * i + 1] = c[i].y;
                     w[4 * i + 2] = c[i].z; w[4 * i + 3] = c[i].w;
                 }
@@ -456,7 +457,7 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                 // balanced-tree sum with a small stack of partial sums (level l holds 2^l terms)
                 V part[6];
 #pragma unroll
-                for (int k = 0; k < NB; ++k) {
+                for (int k = 0; k < NBP; ++k) {
                     V cur;
                     if constexpr (kPermAddr) {
                         const uint32_t sel = static_cast<uint32_t>(k & 3) | (static_cast<uint32_t>(4 + (k & 3)) << 8) | 0x0c0c0000u;
@@ -466,7 +467,7 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                         cur = lds_floats<HPB>(__builtin_amdgcn_perm(wds[k >> 2], pofs4[k >> 2], sel));
                     } else {
                         const uint32_t byte = (wds[k >> 2] >> (8 * (k & 3))) & 0xffu;
-                        cur = *reinterpret_cast<const V*>(ktab_b + byte * (NB * L::ESZ) + pofs[k]);
+                        cur = *reinterpret_cast<const V*>(ktab_b + byte * (NBP * L::ESZ) + pofs[k]);
                     }
 #pragma unroll
                     for (int l = 0; l < 6; ++l) {
@@ -478,42 +479,69 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                             break;
                         }
                     }
-                    if (k == NB - 1) part[5] = cur;
+                    if (k == NBP - 1) part[5] = cur;
                     // keep at most 8 look-ups in flight: bounds the registers this loop needs
                     if ((k & 7) == 7) __builtin_amdgcn_sched_barrier(0);
                 }
-                const V acc = part[5];
-                if constexpr (!MINMAX_ONLY) *reinterpret_cast<V*>(slot(tt)) = acc;
+                V acc = part[5];
+                if constexpr (P > 0) {   // add the earlier pass's partial
+                    const V prev = *reinterpret_cast<const V*>(slot(tt));
 #pragma unroll
-                for (int h = 0; h < HPB; ++h) { mn[h] = fminf(mn[h], acc.v[h]); mx[h] = fmaxf(mx[h], acc.v[h]); }
+                    for (int h = 0; h < HPB; ++h) acc.v[h] += prev.v[h];
+                }
+                if constexpr (!MINMAX_ONLY || P + 1 < L::KPASS) *reinterpret_cast<V*>(slot(tt)) = acc;
+                if constexpr (P + 1 == L::KPASS) {
+#pragma unroll
+                    for (int h = 0; h < HPB; ++h) { mn[h] = fminf(mn[h], acc.v[h]); mx[h] = fmaxf(mx[h], acc.v[h]); }
+                }
             }
         };
-        // first batch: rows already in registers; each consumed round frees registers
-        // that take the first block of packed V rows
-        // (written out round by round with constant indices so vc stays in registers)
-#define CQ_K_ROUND(R)                                                                         \
-        if constexpr (L::KR > (R)) {                                                          \
-            token_logits(tid + (R) * kNT, kc[(R)]);                                           \
-            if constexpr (!MINMAX_ONLY) {                                                     \
-                if constexpr (kVEarly + (R) * BITS < kPF) request_v(kVEarly + (R) * BITS);        \
-                if constexpr (BITS == 2 && kVEarly + (R) * BITS + 1 < kPF) request_v(kVEarly + (R) * BITS + 1); \
-            }                                                                                 \
-        }
-        CQ_K_ROUND(0)
-        CQ_K_ROUND(1)
-        CQ_K_ROUND(2)
-        CQ_K_ROUND(3)
-#undef CQ_K_ROUND
-        static_assert(L::KR <= 4, "rounds are written out up to 4");
-        for (int tb = kNT * L::KR; tb < n; tb += kNT * L::KR) {
+        auto k_pass = [&](auto pass_c) {
+            constexpr int P = decltype(pass_c)::value;
+            // byte table of the pass's positions = high-nibble table + low-nibble table
+            for (int e = tid; e < NBP * 256; e += kNT) {
+                const int j = P * NBP + e % NBP, v = e / NBP;
+                const V hi = nib[(16 + (v >> 4)) * NB + j];
+                const V lo = nib[(v & 15) * NB + j];
+                V o;
 #pragma unroll
-            for (int r = 0; r < L::KR; ++r) {
-                const int tt = min(tb + tid + r * kNT, n - 1);
-#pragma unroll
-                for (int i = 0; i < BITS; ++i) kc[r][i] = ckp[static_cast<int64_t>(tt) * BITS + i];
+                for (int h = 0; h < HPB; ++h) o.v[h] = hi.v[h] + lo.v[h];
+                ktab[e] = o;
             }
+            __syncthreads();
+            // first batch: rows already in registers; each consumed round of the last pass frees
+            // registers that take the first block of packed V rows
+            // (written out round by round with constant indices so vc stays in registers)
+#define CQ_K_ROUND(R)                                                                         \
+            if constexpr (L::KR > (R)) {                                                      \
+                token_logits(pass_c, tid + (R) * kNT, kc[(R)] + P * L::PPP);                  \
+                if constexpr (!MINMAX_ONLY && P + 1 == L::KPASS) {                            \
+                    if constexpr (kVEarly + (R) * BITS < kPF) request_v(kVEarly + (R) * BITS);    \
+                    if constexpr (BITS == 2 && kVEarly + (R) * BITS + 1 < kPF) request_v(kVEarly + (R) * BITS + 1); \
+                }                                                                             \
+            }
+            CQ_K_ROUND(0)
+            CQ_K_ROUND(1)
+            CQ_K_ROUND(2)
+            CQ_K_ROUND(3)
+#undef CQ_K_ROUND
+            static_assert(L::KR <= 4, "rounds are written out up to 4");
+            uint4 kx[L::KR][L::PPP];   // rows beyond the first batch: this pass's pieces only
+            for (int tb = kNT * L::KR; tb < n; tb += kNT * L::KR) {
 #pragma unroll
-            for (int r = 0; r < L::KR; ++r) token_logits(tb + tid + r * kNT, kc[r]);
+                for (int r = 0; r < L::KR; ++r) {
+                    const int tt = min(tb + tid + r * kNT, n - 1);
+#pragma unroll
+                    for (int i = 0; i < L::PPP; ++i) kx[r][i] = ckp[static_cast<int64_t>(tt) * BITS + P * L::PPP + i];
+                }
+#pragma unroll
+                for (int r = 0; r < L::KR; ++r) token_logits(pass_c, tb + tid + r * kNT, kx[r]);
+            }
+        };
+        k_pass(std::integral_constant<int, 0>{});
+        if constexpr (L::KPASS == 2) {
+            __syncthreads();   // every wave is done with the first pass's table
+            k_pass(std::integral_constant<int, 1>{});
         }
     }
     if (n > 0) {   // one reduction for both: max of (-min, max)
@@ -1071,7 +1099,10 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
         else if (G % 2 == 0) vtok ? plan_for<1, 2, true>(a, p) : plan_for<1, 2, false>(a, p);
         else vtok ? plan_for<1, 1, true>(a, p) : plan_for<1, 1, false>(a, p);
     } else {
-        if (G % 2 == 0) vtok ? plan_for<2, 2, true>(a, p) : plan_for<2, 2, false>(a, p);
+        // four heads per unit need the two-pass K table; with per-token values their LDS layout
+        // would not hold a 3 328-token chunk, so that mode keeps two heads per unit
+        if (G % 4 == 0 && !vtok) plan_for<2, 4, false>(a, p);
+        else if (G % 2 == 0) vtok ? plan_for<2, 2, true>(a, p) : plan_for<2, 2, false>(a, p);
         else vtok ? plan_for<2, 1, true>(a, p) : plan_for<2, 1, false>(a, p);
     }
     const int64_t blocks = static_cast<int64_t>(a->B) * a->Hkv * (G / p->hpb) * p->nx;
@@ -1112,8 +1143,9 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
         DecodeGeom g1 = gm;
         g1.nx = g.nsplit;  // the min/max pass has no residual unit
         g1.d_nx.set(static_cast<uint32_t>(g.nsplit));
-        g1.cap = 0;        // ... and keeps no logits
-        const int lds_mm = Lay<BITS, HPB, false>::lds_bytes(0);
+        // ... and keeps no logits, unless the table takes two passes (partial logits wait in the slots)
+        g1.cap = Lay<BITS, HPB, false>::KPASS > 1 ? p.cap : 0;
+        const int lds_mm = Lay<BITS, HPB, false>::lds_bytes(g1.cap);
         hipLaunchKernelGGL(kmm, dim3(units * g.nsplit), dim3(kNT), lds_mm, st, g1);
         CQ_LAUNCH_CHECK();
     }
@@ -1133,6 +1165,9 @@ static int dispatch(const DecodeGeom& g, const Plan& p, int bits, hipStream_t st
         if (p.hpb == 4) return launch<1, 4, DT, VTOK>(g, p, st);
         if (p.hpb == 2) return launch<1, 2, DT, VTOK>(g, p, st);
         return launch<1, 1, DT, VTOK>(g, p, st);
+    }
+    if constexpr (!VTOK) {
+        if (p.hpb == 4) return launch<2, 4, DT, false>(g, p, st);
     }
     if (p.hpb == 2) return launch<2, 2, DT, VTOK>(g, p, st);
     return launch<2, 1, DT, VTOK>(g, p, st);
