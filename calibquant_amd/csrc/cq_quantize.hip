@@ -273,6 +273,7 @@ __global__ __launch_bounds__(kQThreads) void emit_kernel(const uint16_t* __restr
 constexpr int kFThreads = 1024;
 constexpr int kFRows = 13;                  // rows per thread at most (13 x 256 = 12 tiles + thumbnail of 256 tokens)
 constexpr int kFMaxT = kFRows * (kFThreads / 4);
+constexpr int kFGrid = 256;                 // workgroups of the persistent launch (one per compute unit)
 
 template <typename DT, int BITS, int NR>   // NR: rows per thread (T <= NR * 256)
 __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* __restrict__ x, QuantGeom g, float clip,
@@ -285,21 +286,37 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
     __shared__ float s_s[32], s_z[32], s_thr[3][32];
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int q4 = tid & 3, row = tid >> 2;
-    // the four quarters of one (batch, head) sit on one XCD (block ids 8 apart), so the four
-    // 4-byte pieces of a packed row meet in one L2
-    const int quarter = (blockIdx.x >> 3) & 3;
-    const int64_t bh = static_cast<int64_t>(blockIdx.x >> 5) * 8 + (blockIdx.x & 7);
-    if (bh >= static_cast<int64_t>(g.B) * g.H) return;
-    const int b = static_cast<int>(bh / g.H), h = static_cast<int>(bh % g.H);
-    const uint16_t* base = x + b * g.sb + h * g.sh + quarter * 32 + q4 * 8;
-
+    // A workgroup walks slices blockIdx.x, blockIdx.x + gridDim.x, ... (gridDim.x is a multiple
+    // of 32).  The four quarters of one (batch, head) sit on one XCD (slice ids 8 apart), so the
+    // four 4-byte pieces of a packed row meet in one L2.  While a slice's rows are emitted, every
+    // row's registers are refilled with the same row of the next slice: its loads are in flight
+    // during the emit and its min / max pass starts without a wait.
+    const int nslice = static_cast<int>((static_cast<int64_t>(g.B) * g.H + 7) / 8) * 32;
+    const int64_t nbh = static_cast<int64_t>(g.B) * g.H;
+    auto slice_base = [&](int vb) -> const uint16_t* {   // slices past the last (batch, head) alias the last one
+        const int quarter = (vb >> 3) & 3;
+        const int64_t bh = min(static_cast<int64_t>(vb >> 5) * 8 + (vb & 7), nbh - 1);
+        const int b = static_cast<int>(bh / g.H), h = static_cast<int>(bh % g.H);
+        return x + b * g.sb + h * g.sh + quarter * 32 + q4 * 8;
+    };
     typedef uint32_t U4 __attribute__((ext_vector_type(4)));
     U4 v[NR];
+    {
+        const uint16_t* base = slice_base(blockIdx.x);
 #pragma unroll
-    for (int i = 0; i < NR; ++i) {   // rows past T re-read row T-1: min / max unchanged, never written
-        const int t = min(i * (kFThreads / 4) + row, g.T - 1);
-        v[i] = *reinterpret_cast<const U4*>(base + t * g.st);
+        for (int i = 0; i < NR; ++i) {   // rows past T re-read row T-1: min / max unchanged, never written
+            const int t = min(i * (kFThreads / 4) + row, g.T - 1);
+            v[i] = *reinterpret_cast<const U4*>(base + t * g.st);
+        }
     }
+    for (int vb = blockIdx.x; vb < nslice; vb += gridDim.x) {
+    const int quarter = (vb >> 3) & 3;
+    const int64_t bh = static_cast<int64_t>(vb >> 5) * 8 + (vb & 7);
+    const bool live = bh < nbh;                         // a padding slice computes and writes nothing
+    const bool has_next = vb + static_cast<int>(gridDim.x) < nslice;
+    const uint16_t* next_base = slice_base(has_next ? vb + gridDim.x : vb);
+    int row_i = row;   // opaque per iteration: the row offsets below are recomputed, not kept in registers across the loop
+    asm volatile("" : "+v"(row_i));
     float mn[8], mx[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) { mn[j] = INFINITY; mx[j] = -INFINITY; }
@@ -325,7 +342,7 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
         for (int j = 0; j < 8; ++j) { o[j] = mn[j]; o[8 + j] = mx[j]; }
     }
     __syncthreads();
-    if (tid < 32) {   // channel c of the quarter: fold the 64 partials, run the statistics chain
+    if (tid < 32 && live) {   // channel c of the quarter: fold the 64 partials, run the statistics chain
         const int c = tid;
         float a = INFINITY, z = -INFINITY;
 #pragma unroll 4
@@ -378,7 +395,7 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
     constexpr int nb = 128 * BITS / 8;   // bytes per packed row
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
-        const int t = i * (kFThreads / 4) + row;
+        const int t = i * (kFThreads / 4) + row_i;
         // (the empty statement keeps the compiler from carrying the unpacked floats of the
         // min/max pass over to here: that would double the registers the slice needs)
         asm volatile("" : "+v"(v[i]));
@@ -390,7 +407,7 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
             code[j] = (f[j] >= th[0][j]) ? 1u : 0u;
             if constexpr (BITS == 2) code[j] += ((f[j] >= th[1][j]) ? 1u : 0u) + ((f[j] >= th[2][j]) ? 1u : 0u);
         }
-        uint8_t* o = codes + (bh * g.T + min(t, g.T - 1)) * nb + quarter * (nb / 4);
+        uint8_t* o = codes + (min(bh, nbh - 1) * g.T + min(t, g.T - 1)) * nb + quarter * (nb / 4);
         if constexpr (BITS == 1) {
             uint32_t w = 0;
 #pragma unroll
@@ -398,14 +415,17 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
             w <<= 8 * q4;
             w |= static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(w), 0xB1, 0xf, 0xf, true));
             w |= static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(w), 0x4E, 0xf, 0xf, true));
-            if (q4 == 0 && t < g.T) *reinterpret_cast<uint32_t*>(o) = w;
+            if (q4 == 0 && t < g.T && live) *reinterpret_cast<uint32_t*>(o) = w;
         } else {
             const uint32_t b0 = (code[0] << 6) | (code[1] << 4) | (code[2] << 2) | code[3];
             const uint32_t b1 = (code[4] << 6) | (code[5] << 4) | (code[6] << 2) | code[7];
             const uint32_t half = b0 | (b1 << 8);
             const uint32_t other = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(half), 0xB1, 0xf, 0xf, true));
-            if ((q4 & 1) == 0 && t < g.T) reinterpret_cast<uint32_t*>(o)[q4 >> 1] = half | (other << 16);
+            if ((q4 & 1) == 0 && t < g.T && live) reinterpret_cast<uint32_t*>(o)[q4 >> 1] = half | (other << 16);
         }
+        // the row is packed: its registers take the same row of the next slice
+        if (has_next) v[i] = *reinterpret_cast<const U4*>(next_base + min(t, g.T - 1) * g.st);
+    }
     }
 }
 
@@ -419,7 +439,9 @@ static int run_quant(const void* x, QuantGeom g, int bits, float clip, uint8_t* 
     if (!xq && g.D == 128 && g.T <= kFMaxT && (reinterpret_cast<uintptr_t>(codes) & 3u) == 0) {
         // x fits a workgroup's registers slice by slice: one pass
         const int64_t bh8 = (static_cast<int64_t>(g.B) * g.H + 7) / 8;
-        const dim3 fgrid(static_cast<unsigned>(bh8 * 32));
+        // persistent: at most one workgroup per compute unit and a multiple of 32 of them
+        const int64_t nsl = bh8 * 32;
+        const dim3 fgrid(static_cast<unsigned>(nsl < kFGrid ? nsl : kFGrid));
         const int nr = (g.T + kFThreads / 4 - 1) / (kFThreads / 4);
 #define CQ_FUSED(B_, N_) hipLaunchKernelGGL((fused_pack_kernel<DT, B_, N_>), fgrid, dim3(kFThreads), 0, st, xp, g, clip, sp, zp, codes)
         if (bits == 1) {
