@@ -90,6 +90,19 @@ __device__ __forceinline__ void store_elem(void* p, int64_t i, float f) {
     static_cast<uint16_t*>(p)[i] = static_cast<uint16_t>(Cvt<DT>::from_float(f));
 }
 
+// Division of indices (< 2^31) by a small run-time constant without the integer-division
+// expansion: q = (mulhi(n, mul) + n) >> shift, with mul and shift worked out on the host.
+struct FastDiv {
+    uint32_t mul, shift, div;
+    __host__ void set(uint32_t d) {
+        div = d;
+        shift = 0;
+        while ((1u << shift) < d) ++shift;
+        mul = static_cast<uint32_t>(((static_cast<uint64_t>(1) << 32) * ((static_cast<uint64_t>(1) << shift) - d)) / d + 1);
+    }
+    __device__ __forceinline__ uint32_t quot(uint32_t n) const { return (__umulhi(n, mul) + n) >> shift; }
+};
+
 // ------------------------------------------------------- wave reductions
 // Cross-lane moves use the data-parallel-primitive modifiers of the VALU (no LDS
 // traffic, one instruction per step).  Control codes: quad_perm[1,0,3,2] = 0xB1,

@@ -49,19 +49,6 @@ template <int N> struct alignas(N * 4) Vec { float v[N]; };
 // native 16-byte vector: copies are single vector moves (HIP's uint4 struct copies lower to memcpy)
 typedef uint32_t U4 __attribute__((ext_vector_type(4)));
 
-// Division of block indices (< 2^31) by a small run-time constant without the integer-division
-// expansion: q = (mulhi(n, mul) + n) >> shift, with mul and shift worked out on the host.
-struct FastDiv {
-    uint32_t mul, shift, div;
-    __host__ void set(uint32_t d) {
-        div = d;
-        shift = 0;
-        while ((1u << shift) < d) ++shift;
-        mul = static_cast<uint32_t>(((static_cast<uint64_t>(1) << 32) * ((static_cast<uint64_t>(1) << shift) - d)) / d + 1);
-    }
-    __device__ __forceinline__ uint32_t quot(uint32_t n) const { return (__umulhi(n, mul) + n) >> shift; }
-};
-
 struct DecodeGeom {
     const void* q;
     const uint8_t* ck;

@@ -29,6 +29,7 @@ struct QuantGeom {
     int B, T, H, D;
     int64_t sb, st, sh;   // element strides of x
     int nchunk, chunk;    // token chunks
+    FastDiv dT, dH;       // divisors T and H of a flat (b, h, t) row index (per-token quantiser)
 };
 
 static inline int pick_chunks(int B, int T, int H) {
@@ -488,7 +489,7 @@ static int quant_entry(const void* x, int dtype, int B, int T, int H, int D, int
         return CQ_ERR_ALIGN;
     const size_t need = cq_quantize_pack_workspace(B, T, H, D);
     if (!ws || ws_bytes < need || !aligned16(ws)) return CQ_ERR_WORKSPACE;
-    QuantGeom g;
+    QuantGeom g = {};
     g.B = B; g.T = T; g.H = H; g.D = D;
     g.sb = sb; g.st = st; g.sh = sh;
     g.nchunk = pick_chunks(B, T, H);
@@ -521,10 +522,21 @@ __global__ __launch_bounds__(kQThreads) void token_pack_kernel(const uint16_t* _
     const float inv_levels = __fdiv_rn(1.0f, levels);
     for (int64_t row = blockIdx.x * static_cast<int64_t>(kQThreads / 16) + (threadIdx.x >> 4); row < rows;
          row += static_cast<int64_t>(gridDim.x) * (kQThreads / 16)) {
-        // output row order (b, h, t)
-        const int t = static_cast<int>(row % g.T);
-        const int h = static_cast<int>((row / g.T) % g.H);
-        const int b = static_cast<int>(row / (static_cast<int64_t>(g.T) * g.H));
+        // output row order (b, h, t); row indices below 2^31 are split with host-prepared
+        // multipliers instead of 64-bit divisions
+        int t, h, b;
+        if (rows < (static_cast<int64_t>(1) << 31)) {
+            const uint32_t r32 = static_cast<uint32_t>(row);
+            const uint32_t bh = g.dT.quot(r32);
+            t = static_cast<int>(r32 - bh * g.dT.div);
+            const uint32_t bq = g.dH.quot(bh);
+            h = static_cast<int>(bh - bq * g.dH.div);
+            b = static_cast<int>(bq);
+        } else {
+            t = static_cast<int>(row % g.T);
+            h = static_cast<int>((row / g.T) % g.H);
+            b = static_cast<int>(row / (static_cast<int64_t>(g.T) * g.H));
+        }
         const uint4 v = *reinterpret_cast<const uint4*>(x + b * g.sb + t * g.st + h * g.sh + l16 * 8);
         float f[8];
         unpack8<DT>(v, f);
@@ -650,10 +662,12 @@ int cq_quantize_pack_token(const void* x, int dtype, int B, int T, int H, int D,
         (reinterpret_cast<uintptr_t>(words) & 3u) || (reinterpret_cast<uintptr_t>(scale) & 1u) ||
         (reinterpret_cast<uintptr_t>(mins) & 1u))
         return CQ_ERR_ALIGN;
-    cq::QuantGeom g;
+    cq::QuantGeom g = {};
     g.B = B; g.T = T; g.H = H; g.D = D;
     g.sb = stride_b; g.st = stride_t; g.sh = stride_h;
     g.nchunk = 1; g.chunk = T;
+    g.dT.set(static_cast<uint32_t>(T));
+    g.dH.set(static_cast<uint32_t>(H));
     const int64_t rows = static_cast<int64_t>(B) * H * T;
     int64_t blocks = (rows + cq::kQThreads / 16 - 1) / (cq::kQThreads / 16);
     if (blocks > (1 << 20)) blocks = 1 << 20;
