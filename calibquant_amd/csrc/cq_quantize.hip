@@ -296,9 +296,9 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
     const int64_t nbh = static_cast<int64_t>(g.B) * g.H;
     auto slice_base = [&](int vb) -> const uint16_t* {   // slices past the last (batch, head) alias the last one
         const int quarter = (vb >> 3) & 3;
-        const int64_t bh = min(static_cast<int64_t>(vb >> 5) * 8 + (vb & 7), nbh - 1);
-        const int b = static_cast<int>(bh / g.H), h = static_cast<int>(bh % g.H);
-        return x + b * g.sb + h * g.sh + quarter * 32 + q4 * 8;
+        const uint32_t bh = static_cast<uint32_t>(min(static_cast<int64_t>(vb >> 5) * 8 + (vb & 7), nbh - 1));
+        const uint32_t b = g.dH.quot(bh), h = bh - b * g.dH.div;   // B * H < 2^31 on this path
+        return x + static_cast<int64_t>(b) * g.sb + static_cast<int64_t>(h) * g.sh + quarter * 32 + q4 * 8;
     };
     typedef uint32_t U4 __attribute__((ext_vector_type(4)));
     U4 v[NR];
@@ -437,7 +437,8 @@ static int run_quant(const void* x, QuantGeom g, int bits, float clip, uint8_t* 
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     uint16_t* sp = static_cast<uint16_t*>(scale);
     uint16_t* zp = static_cast<uint16_t*>(zero);
-    if (!xq && g.D == 128 && g.T <= kFMaxT && (reinterpret_cast<uintptr_t>(codes) & 3u) == 0) {
+    if (!xq && g.D == 128 && g.T <= kFMaxT && (reinterpret_cast<uintptr_t>(codes) & 3u) == 0 &&
+        static_cast<int64_t>(g.B) * g.H < (static_cast<int64_t>(1) << 31)) {
         // x fits a workgroup's registers slice by slice: one pass
         const int64_t bh8 = (static_cast<int64_t>(g.B) * g.H + 7) / 8;
         // persistent: at most one workgroup per compute unit and a multiple of 32 of them
@@ -494,6 +495,8 @@ static int quant_entry(const void* x, int dtype, int B, int T, int H, int D, int
     g.sb = sb; g.st = st; g.sh = sh;
     g.nchunk = pick_chunks(B, T, H);
     g.chunk = (T + g.nchunk - 1) / g.nchunk;
+    g.dT.set(static_cast<uint32_t>(T));
+    g.dH.set(static_cast<uint32_t>(H));
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == CQ_BF16)
         return run_quant<BF16>(x, g, bits, clip, codes, xq, scale, zero, static_cast<float*>(ws), s);
