@@ -127,6 +127,27 @@ def time_fp16_kv(torch, shape, steps, warmup, nsets):
     return start.elapsed_time(end) / steps
 
 
+def time_fp16_kv_own(torch, ops, shape, steps, warmup, nsets):
+    """Full-precision-KV attention over the same tokens with this library's own kernel: every
+    token a row of the full-precision window (no packed part)."""
+    B, Hq, Hkv, D, T, R, S = shape
+    dev = torch.device("cuda:0")
+    N = T + R
+    calls = []
+    for _ in range(nsets):
+        q = torch.randn((B, Hq, D), device=dev, dtype=torch.bfloat16)
+        k = torch.randn((B, Hkv, N, D), device=dev, dtype=torch.bfloat16)
+        v = torch.randn((B, Hkv, N, D), device=dev, dtype=torch.bfloat16)
+        calls.append(ops.DecodeCall(q, None, None, None, None, None, None, k, v, sprompt_len=0, bits=1))
+    it = [0]
+
+    def run():
+        calls[it[0] % nsets].run()
+        it[0] += 1
+
+    return _time_fn(torch, run, steps, warmup)
+
+
 def _time_fn(torch, fn, steps, warmup):
     for _ in range(warmup):
         fn()
@@ -262,7 +283,7 @@ def model_leg(torch, batch=64, tiles=13, sys_len=41, text_len=23, new_tokens=128
         res[tag + "_eager_ms_per_token_step"] = round(dt / (new_tokens - 1) * 1e3, 3)
         drop_state()
 
-    def run_graph(tag, patched):
+    def run_graph(tag, patched, fp_kernel=False):
         """The decode step recorded once as a HIP graph and replayed per token; timed over the
         replays only (the first decode step runs eagerly and the recording follows it)."""
         from calibquant_amd.graph_decode import StaticDecoder
@@ -286,7 +307,7 @@ def model_leg(torch, batch=64, tiles=13, sys_len=41, text_len=23, new_tokens=128
             logits, past = lm.forward_step(emb, pos, None)
             del emb, vit
             first = logits[:, -1].argmax(-1)
-            dec = StaticDecoder(lm, past, N, new_tokens)
+            dec = StaticDecoder(lm, past, N, new_tokens, fp_kernel=fp_kernel)
             del past
             drop_state()
             out = dec.generate(first, new_tokens, use_graph=True, on_step=on_step)
@@ -304,6 +325,9 @@ def model_leg(torch, batch=64, tiles=13, sys_len=41, text_len=23, new_tokens=128
         # length mask - what a recorded step would need - falls back to a much slower kernel.
         run_eager("fp16_kv", False)
         res["fp16_kv_decode_tok_s"] = res["fp16_kv_eager_decode_tok_s"]
+        # ... and the same full-precision cache read by this library's own attention kernel (every
+        # token a row of its full-precision window), step recorded as a HIP graph: the stronger baseline
+        run_graph("fp16_kv_own_kernel", False, fp_kernel=True)
         import contextlib, io
         with contextlib.redirect_stdout(io.StringIO()):
             pi.patch_model(model, "calibquant")
@@ -312,7 +336,8 @@ def model_leg(torch, batch=64, tiles=13, sys_len=41, text_len=23, new_tokens=128
     finally:
         InternLM2Attention.forward, InternVLChatStandIn.generate = fp_forward, fp_generate
     res["note"] = ("kv_1bit_decode_tok_s: decode step replayed as a HIP graph; *_eager_*: eager host loop "
-                   "(1-bit: bound by per-layer launch overhead; fp16: bound by the attention kernel)")
+                   "(1-bit: bound by per-layer launch overhead; fp16: torch SDPA, bound by that attention kernel); "
+                   "fp16_kv_own_kernel_*: full-precision cache through this library's attention kernel, HIP graph")
     return res
 
 
@@ -383,6 +408,9 @@ def main():
             fp_ms = time_fp16_kv(torch, shape, max(20, a.steps // 4), max(5, a.warmup // 4), a.sets)
             out["fp16_kv_us_layer"] = round(fp_ms * 1e3, 2)
             out["speedup_vs_fp16_kv"] = round(fp_ms / ms, 2)
+            own_ms = time_fp16_kv_own(torch, ops, shape, max(20, a.steps // 4), max(5, a.warmup // 4), a.sets)
+            out["fp16_kv_own_kernel_us_layer"] = round(own_ms * 1e3, 2)
+            out["speedup_vs_fp16_kv_own_kernel"] = round(own_ms / ms, 2)
         except Exception as e:  # the comparison leg must not sink the measurement
             out["fp16_kv_us_layer"] = None
             out["fp16_kv_error"] = repr(e)[:200]

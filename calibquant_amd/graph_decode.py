@@ -13,8 +13,10 @@ the attention kernel reads the row count on the device
 
 Two variants share the step: attention modules patched by
 `patch_internvl.patch_model` run the packed-KV kernel; unpatched modules keep
-a full-precision cache and use torch's scaled-dot-product attention over the
-whole buffer with a length mask computed on the device.
+a full-precision cache and use either torch's scaled-dot-product attention over
+the whole buffer with a length mask computed on the device, or (`fp_kernel=True`)
+this library's attention kernel with every cached token as a row of its
+full-precision window.
 """
 from __future__ import annotations
 
@@ -31,7 +33,8 @@ from .patch_internvl import CALIB_OFFSET_MAX, CALIB_OFFSET_MIN
 class _LayerState:
     """Fixed-address decode state of one attention module."""
 
-    def __init__(self, att, past, capacity: int, r_len: torch.Tensor, quantized: bool, cos, sin, pos, row):
+    def __init__(self, att, past, capacity: int, r_len: torch.Tensor, quantized: bool, cos, sin, pos, row,
+                 fp_kernel: bool = False):
         k_old, v_old = past
         B, Hkv, R0, D = k_old.shape
         self.quantized = quantized
@@ -58,6 +61,9 @@ class _LayerState:
                                        bits=att.bits_k, calibrate=att.normalize, calib_off_max=CALIB_OFFSET_MAX,
                                        calib_off_min=CALIB_OFFSET_MIN, out=self.out, r_dev=r_len,
                                        v_mode=getattr(att, "v_mode", "channel"))
+        elif fp_kernel:
+            self.call = ops.DecodeCall(self.q, None, None, None, None, None, None, self.kbuf, self.vbuf,
+                                       sprompt_len=0, bits=1, out=self.out, r_dev=r_len)
 
 
 class StaticDecoder:
@@ -68,7 +74,7 @@ class StaticDecoder:
     the whole cache otherwise); prompt_len: tokens in the prompt (the position
     of the first generated token); logits: the prefill's last-position logits."""
 
-    def __init__(self, lm, past, prompt_len: int, max_new_tokens: int):
+    def __init__(self, lm, past, prompt_len: int, max_new_tokens: int, fp_kernel: bool = False):
         layers = lm.model.layers
         att0 = layers[0].attention
         self.lm = lm
@@ -89,7 +95,7 @@ class StaticDecoder:
         self.cos, self.sin = cos.contiguous(), sin.contiguous()
         self.state: List[_LayerState] = [
             _LayerState(l.attention, past[i], self.capacity, self.r_len, self.quantized, self.cos, self.sin,
-                        self.pos, self.r_idx) for i, l in enumerate(layers)]
+                        self.pos, self.r_idx, fp_kernel) for i, l in enumerate(layers)]
         self.col = torch.arange(self.capacity, device=dev)
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.steps_left = max_new_tokens
@@ -104,7 +110,7 @@ class StaticDecoder:
             h = F.rms_norm(x, (x.shape[-1],), layer.attention_norm.weight, layer.attention_norm.eps)
             torch.matmul(h.view(B, -1), att.wqkv.weight.t(), out=st.qkv)
             st.rope.run()            # st.q <- rotated query heads; window row r_idx <- rotated key, value
-            if st.quantized:
+            if st.call is not None:
                 st.call.run()
                 o = st.out
             else:

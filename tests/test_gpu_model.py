@@ -170,8 +170,8 @@ def _prefill(m, ids, pix=None):
     return lm.forward_step(emb, pos, None)
 
 
-@pytest.mark.parametrize("quantized", [True, False])
-def test_static_decoder_graph_replays_equal_eager_steps(quantized):
+@pytest.mark.parametrize("quantized,fp_kernel", [(True, False), (False, False), (False, True)])
+def test_static_decoder_graph_replays_equal_eager_steps(quantized, fp_kernel):
     """The recorded decode step, replayed per token, produces the tokens of the same step run
     eagerly, and its first step agrees with the model's own eager step."""
     from calibquant_amd import patch_internvl as pi
@@ -196,7 +196,7 @@ def test_static_decoder_graph_replays_equal_eager_steps(quantized):
             for use_graph in (False, True):
                 logits, past = _prefill(m, ids, pix)
                 first = logits[:, -1].argmax(-1)
-                dec = StaticDecoder(lm, past, N, NEW)
+                dec = StaticDecoder(lm, past, N, NEW, fp_kernel=fp_kernel)
                 toks = dec.generate(first, NEW, use_graph=use_graph)
                 torch.cuda.synchronize()
                 assert (dec.graph is not None) == use_graph
@@ -206,7 +206,7 @@ def test_static_decoder_graph_replays_equal_eager_steps(quantized):
             # same arithmetic up to rounding)
             logits, past = _prefill(m, ids, pix)
             first = logits[:, -1].argmax(-1)
-            dec = StaticDecoder(lm, past, N, 2)
+            dec = StaticDecoder(lm, past, N, 2, fp_kernel=fp_kernel)
             dec.tok.copy_(first)
             x = lm.get_input_embeddings()(first)[:, None]
             pos1 = torch.full((B, 1), N, device="cuda", dtype=torch.long)
