@@ -220,7 +220,7 @@ def cpu_baseline(torch, sets, shape, bits, budget_s=12.0):
                       f"scaled x{B // bs} to the full batch"}
 
 
-def model_leg(torch, batch=64, tiles=13, sys_len=41, text_len=23, new_tokens=128, seed=1234):
+def model_leg(torch, batch=64, tiles=13, sys_len=41, text_len=23, new_tokens=128, seed=1234, model_name="8b"):
     """InternVL2.5-8B-shaped decode (InternLM2.5-7B language model: 32 layers, hidden 4096, 32/8
     heads, head_dim 128, vocab 92 553), random-init bf16 weights, synthetic uniform-noise tiles
     through a stand-in vision tower: tokens/s of `new_tokens` greedy steps at `batch`, prefill
@@ -233,7 +233,8 @@ def model_leg(torch, batch=64, tiles=13, sys_len=41, text_len=23, new_tokens=128
     torch.set_default_dtype(torch.bfloat16)
     try:
         with torch.device(dev):
-            model = InternVLChatStandIn(InternLM2Config.internvl2_5_8b()).eval()
+            cfg = InternLM2Config.internvl2_5_26b() if model_name == "26b" else InternLM2Config.internvl2_5_8b()
+            model = InternVLChatStandIn(cfg).eval()
     finally:
         torch.set_default_dtype(prev)
     T = tiles * 256
@@ -241,7 +242,8 @@ def model_leg(torch, batch=64, tiles=13, sys_len=41, text_len=23, new_tokens=128
     ids = torch.randint(0, 90000, (batch, N), device=dev)
     ids[:, sys_len:sys_len + T] = model.img_context_token_id
     fp_forward, fp_generate = InternLM2Attention.forward, InternVLChatStandIn.generate
-    res = {"prompt_tokens": N, "image_tokens": T, "new_tokens": new_tokens, "batch": batch}
+    res = {"model": "internvl2.5-" + model_name + "-shaped", "prompt_tokens": N, "image_tokens": T,
+           "new_tokens": new_tokens, "batch": batch}
 
     def features():
         vis = []
@@ -352,6 +354,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-fp16kv", action="store_true", help="skip the fp16-KV comparison leg")
     ap.add_argument("--no-model", action="store_true", help="skip the full-model decode tok/s leg")
+    ap.add_argument("--model", default="8b", choices=("8b", "26b"),
+                    help="language-model shape of the full-model leg (26b: 48 layers, hidden 6144, 48/8 heads)")
     ap.add_argument("--no-side", action="store_true", help="skip the prefill / per-token-value side figures")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch three 256 MiB device copies (known traffic, for scaling profiler byte counters)")
@@ -425,7 +429,10 @@ def main():
         del sets, calls
         torch.cuda.empty_cache()
         try:
-            out["model_decode"] = model_leg(torch)
+            if a.model == "26b":   # InternLM2-20B-shaped: 3 images = 39 tiles, 41 + 23 text tokens, batch 16, 64 new tokens
+                out["model_decode"] = model_leg(torch, batch=16, tiles=39, new_tokens=64, model_name="26b")
+            else:
+                out["model_decode"] = model_leg(torch)
         except Exception as e:  # the model leg must not sink the kernel measurement
             out["model_decode"] = {"error": repr(e)[:300]}
     print(json.dumps(out))
