@@ -355,3 +355,25 @@ def test_decode_attention_per_token_values_brute_force():
             vals += [float(s[0, 0, t, 0]) * int(codes[0, 0, t, d]) + float(mn[0, 0, t, 0]) for t in range(6)]
             vals += [float(vr[0, 0, 1, d])]
             assert abs(out[0, h, d] - sum(pp * vv for pp, vv in zip(p, vals))) < 1e-9
+
+
+def test_oracle_results_are_frozen_by_the_committed_digests():
+    """The oracle's own results on three small seeded cases equal the committed digests
+    (tests/golden/oracle_vectors.json, written by tests/golden/make_vectors.py): an edit that
+    changes the oracle's numbers fails here.  These are not reference outputs."""
+    import importlib.util
+    import json
+    import os
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    spec = importlib.util.spec_from_file_location("make_vectors", os.path.join(here, "make_vectors.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    want = json.load(open(os.path.join(here, "oracle_vectors.json")))
+    got = mod.vectors()
+    assert sorted(got) == sorted(want)
+    for name, w in want.items():
+        g = got[name]
+        for key in ("codes_k", "codes_v", "k_scale", "k_zero", "v_scale", "v_zero"):
+            assert g[key] == w[key], (name, key)
+        assert np.allclose(g["out_head0"], w["out_head0"], atol=2e-6), name
+        assert abs(g["out_sum"] - w["out_sum"]) < 1e-3, name
