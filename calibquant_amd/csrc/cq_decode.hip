@@ -289,27 +289,27 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
     const uint4* cvp = reinterpret_cast<const uint4*>((has_img ? g.cv : static_cast<const uint8_t*>(g.q)) + code_off);
     const U4* cvp4 = reinterpret_cast<const U4*>(cvp);
     const int last_u = has_img ? n * NB / 16 - 1 : 0;   // last valid 16-byte unit of either stream
-    // residual tile: K slice (row = tid/8, 16 elements) and V slices (two rows, 8 elements)
+    // residual tile: K slice (row = tid/8, 16 elements); V: a wave owns 8 rows of the tile and a
+    // lane one channel pair of each of them, so the value products need no fold inside the wave
     const int l8 = tid & 7, krow = tid >> 3;
-    // residual V: lane = (8-element slice ds, row slot): the slot's two low bits sit in the
-    // two low lane bits so the final fold over slots is a quad permute
-    const int ds = (tid >> 2) & 15, rslot = (tid & 3) | ((tid >> 6) << 2);
+    const int wvr = __builtin_amdgcn_readfirstlane(wv);   // wave-uniform: scalar row arithmetic
     const int64_t res_off = do_res ? b * g.rs_b + hkv * g.rs_h : 0;   // one offset for both windows
     const uint16_t* kb = static_cast<const uint16_t*>(do_res ? g.kres : g.q) + res_off;
     const uint16_t* vbp = static_cast<const uint16_t*>(do_res ? g.vres : g.q) + res_off;
     const int last_r = do_res ? R - 1 : 0;
     const int64_t rs_r = do_res ? g.rs_r : 0;
-    uint4 rk[2], rv[2];
+    uint4 rk[2];
+    uint32_t rv[8];
     auto load_res_k = [&](int r0, uint4* k2) {   // rows past R re-read row R-1 (their logit is masked)
         const uint16_t* kp = kb + min(r0 + krow, last_r) * rs_r;
         k2[0] = *reinterpret_cast<const uint4*>(kp + l8 * 8);
         k2[1] = *reinterpret_cast<const uint4*>(kp + 64 + l8 * 8);
     };
-    auto load_res_v = [&](int r0, uint4* v2) {   // rows past R re-read row R-1 (their weight is 0)
+    auto load_res_v = [&](int r0, uint32_t* v8) {   // rows past R re-read row R-1 (their weight is 0)
 #pragma unroll
-        for (int rep = 0; rep < 2; ++rep) {
-            const int r2 = min(r0 + rslot + rep * (kResTile / 2), last_r);
-            v2[rep] = *reinterpret_cast<const uint4*>(vbp + r2 * rs_r + ds * 8);
+        for (int i = 0; i < 8; ++i) {
+            const int r2 = min(r0 + wvr * 8 + i, last_r);
+            v8[i] = *reinterpret_cast<const uint32_t*>(vbp + r2 * rs_r + 2 * lane);
         }
     };
 
@@ -899,9 +899,9 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
             float* pres = fx + L::F_PRES;
             // raw 16-bit q, [head][kD], read per head as two 16-byte LDS loads
             const uint4* q128 = reinterpret_cast<const uint4*>(fx + L::F_QRAW);
-            float accv[8][HPB];
+            float accv[2][HPB];   // the lane's channel pair
 #pragma unroll
-            for (int k = 0; k < 8; ++k)
+            for (int k = 0; k < 2; ++k)
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) accv[k][h] = 0.f;
             const float* mk = g.mask ? g.mask + b * g.mask_sb : nullptr;
@@ -945,35 +945,33 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                     if (lane == 0) { stat[h] = al; stat[HPB + h] = m_run; stat[2 * HPB + h] = l_run; }
                 }
                 __syncthreads();
-                float alpha[HPB];
+                if (r0 > 0) {
 #pragma unroll
-                for (int h = 0; h < HPB; ++h) alpha[h] = stat[h];
-#pragma unroll
-                for (int rep = 0; rep < 2; ++rep) {
-                    const int rr = rslot + rep * (kResTile / 2);
-                    float f[8];
-                    unpack8<DT>(rv[rep], f);
-                    const V p = reinterpret_cast<const V*>(pres)[rr];   // 0 for rows past R
-#pragma unroll
-                    for (int k = 0; k < 8; ++k)
-#pragma unroll
-                        for (int h = 0; h < HPB; ++h)
-                            accv[k][h] = ((rep == 0 && r0 > 0) ? accv[k][h] * alpha[h] : accv[k][h]) + p.v[h] * f[k];
+                    for (int h = 0; h < HPB; ++h) {
+                        const float al = stat[h];
+                        accv[0][h] *= al;
+                        accv[1][h] *= al;
+                    }
                 }
-                if (more) load_res_v(r0 + kResTile, rv);   // next tile's V slices, in place
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float f0 = Cvt<DT>::lo(rv[i]), f1 = Cvt<DT>::hi(rv[i]);
+                    const V p = reinterpret_cast<const V*>(pres)[wvr * 8 + i];   // the row's weights (0 past R), one address per wave
+#pragma unroll
+                    for (int h = 0; h < HPB; ++h) {
+                        accv[0][h] = __builtin_fmaf(p.v[h], f0, accv[0][h]);
+                        accv[1][h] = __builtin_fmaf(p.v[h], f1, accv[1][h]);
+                    }
+                }
+                if (more) load_res_v(r0 + kResTile, rv);   // next tile's V words, in place
             }
-            // fold the row slots: 4 per wave (lane bits 4,5), then the waves
-#pragma unroll
-            for (int k = 0; k < 8; ++k)
-#pragma unroll
-                for (int h = 0; h < HPB; ++h) accv[k][h] = quad_reduce(accv[k][h], OpSum(), 0.f);
             __syncthreads();
             float* red2 = reinterpret_cast<float*>(regA);  // [wave][head][kD]: the fold reads consecutive words
-            if ((lane & 3) == 0) {
 #pragma unroll
-                for (int k = 0; k < 8; ++k)
-#pragma unroll
-                    for (int h = 0; h < HPB; ++h) red2[(wv * HPB + h) * kD + ds * 8 + k] = accv[k][h];
+            for (int h = 0; h < HPB; ++h) {
+                Vec<2> a2;
+                a2.v[0] = accv[0][h]; a2.v[1] = accv[1][h];
+                *reinterpret_cast<Vec<2>*>(red2 + (wv * HPB + h) * kD + 2 * lane) = a2;
             }
             __syncthreads();
             if (tid < HPB * kD) {
