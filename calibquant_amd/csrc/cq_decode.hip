@@ -221,7 +221,9 @@ template <int N> __device__ __forceinline__ Vec<N> lds_floats(uint32_t addr) {
 }
 
 __device__ __forceinline__ uint32_t pack_f16(float a, float b) {
-    f16x2_t h = {static_cast<_Float16>(a), static_cast<_Float16>(b)};   // round to nearest even
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t v = {a, b};
+    const f16x2_t h = __builtin_convertvector(v, f16x2_t);   // one packed conversion, round to nearest even
     return __builtin_bit_cast(uint32_t, h);
 }
 
@@ -662,6 +664,8 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                     const V w = *reinterpret_cast<const V*>(slot(tt));
 #pragma unroll
                     for (int h = 0; h < HPB; ++h) {
+                        // (w - mn) first: with a degenerate logit range the slope is ~1e8 and only the exact
+                        // zero of the difference keeps the product finite
                         e[h] = __builtin_amdgcn_exp2f((w.v[h] - mn[h]) * ea[h] + ec[h]);
                         ls[h] += e[h];
                     }
