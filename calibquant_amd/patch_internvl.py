@@ -219,24 +219,32 @@ def forward_internlm2_calibquant(self, hidden_states: torch.Tensor, attention_ma
             raise ValueError(f"Attention mask should be of size {(bsz, 1, q_len, kv_seq_len)}, "
                              f"but is {attention_mask.size()}")
         mask = attention_mask[:, 0, 0, :]
-    q1 = query_states[:, :, 0, :]
+    out = _attend(self, query_states[:, :, 0, :], k_res, v_res, mask)
+    attn_output = self.wo(out.reshape(bsz, 1, self.hidden_size))
+    return attn_output, None, past_key_value
+
+
+def _attend(self, q1, k_res, v_res, mask):
+    """The fused decode attention of one step over the module's packed state and the full-precision
+    window (k_res, v_res): q1 (B, Hq, D) -> (B, Hq, D).  In the steady state (no mask, same batch and
+    dtype, no workspace) the prepared call of the previous step is re-aimed at this step's tensors."""
+    bsz = q1.shape[0]
+    S, T = self.sprompt_len, self.image_token_num
+    R = k_res.shape[2]
     call = getattr(self, "_cq_call", None)
     if (mask is None and call is not None and call.args.B == bsz and call.workspace_bytes == 0
             and q1.is_contiguous() and call.args.dtype == (0 if q1.dtype == torch.bfloat16 else 1)):
-        # steady state: re-aim the prepared call (same packed state) at this step's tensors
-        out = call.step(q1, k_res, v_res, torch.empty_like(q1))
-    else:
-        stats = self._cq_stats if T > 0 else (None,) * 4
-        call = ops.DecodeCall(q1, self.encoded_features_k if T > 0 else None,
-                              self.encoded_features_v if T > 0 else None, stats[0], stats[1], stats[2], stats[3],
-                              k_res, v_res, sprompt_len=min(S, R), bits=self.bits_k, calibrate=self.normalize,
-                              calib_off_max=CALIB_OFFSET_MAX, calib_off_min=CALIB_OFFSET_MIN, mask=mask,
-                              v_mode=self.v_mode)
-        with torch.cuda.device(call.device):
-            out = call.run()
-        self._cq_call = call if mask is None else None
-    attn_output = self.wo(out.reshape(bsz, 1, self.hidden_size))
-    return attn_output, None, past_key_value
+        return call.step(q1, k_res, v_res, torch.empty_like(q1))
+    stats = self._cq_stats if T > 0 else (None,) * 4
+    call = ops.DecodeCall(q1, self.encoded_features_k if T > 0 else None,
+                          self.encoded_features_v if T > 0 else None, stats[0], stats[1], stats[2], stats[3],
+                          k_res, v_res, sprompt_len=min(S, R), bits=self.bits_k, calibrate=self.normalize,
+                          calib_off_max=CALIB_OFFSET_MAX, calib_off_min=CALIB_OFFSET_MIN, mask=mask,
+                          v_mode=self.v_mode)
+    with torch.cuda.device(call.device):
+        out = call.run()
+    self._cq_call = call if mask is None else None
+    return out
 
 
 def _decode_step_fused(self, qkv, position_ids, past_key_value, attention_mask, use_cache):
@@ -280,20 +288,7 @@ def _decode_step_fused(self, qkv, position_ids, past_key_value, attention_mask, 
             raise ValueError(f"Attention mask should be of size {(bsz, 1, 1, kv_seq_len)}, "
                              f"but is {attention_mask.size()}")
         mask = attention_mask[:, 0, 0, :]
-    call = getattr(self, "_cq_call", None)
-    if (mask is None and call is not None and call.args.B == bsz and call.workspace_bytes == 0
-            and call.args.dtype == (0 if q1.dtype == torch.bfloat16 else 1)):
-        out = call.step(q1, k_res, v_res, torch.empty_like(q1))
-    else:
-        stats = self._cq_stats if T > 0 else (None,) * 4
-        call = ops.DecodeCall(q1, self.encoded_features_k if T > 0 else None,
-                              self.encoded_features_v if T > 0 else None, stats[0], stats[1], stats[2], stats[3],
-                              k_res, v_res, sprompt_len=min(S, R), bits=self.bits_k, calibrate=self.normalize,
-                              calib_off_max=CALIB_OFFSET_MAX, calib_off_min=CALIB_OFFSET_MIN, mask=mask,
-                              v_mode=self.v_mode)
-        with torch.cuda.device(call.device):
-            out = call.run()
-        self._cq_call = call if mask is None else None
+    out = _attend(self, q1, k_res, v_res, mask)
     return self.wo(out.reshape(bsz, 1, self.hidden_size)), None, past_key_value
 
 
