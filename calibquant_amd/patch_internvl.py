@@ -254,7 +254,7 @@ def _decode_step_fused(self, qkv, position_ids, past_key_value, attention_mask, 
     bsz = qkv.shape[0]
     G, D, Hq = self.num_key_value_groups, self.head_dim, self.num_heads
     Hkv = Hq // G
-    S, T = self.sprompt_len, self.image_token_num
+    T = self.image_token_num
     R0 = past_key_value[0].shape[2]
     R = R0 + 1
     kv_seq_len = R + T
