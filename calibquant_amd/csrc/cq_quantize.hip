@@ -363,29 +363,35 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
         s_z[c] = zp;
     }
     __syncthreads();
-    // thresholds (see the statistics kernel): one 64-ary search per (channel, level) and wave,
-    // three rounds narrow the 2^16 ordered storage values down to one.  The code is a
-    // non-decreasing function of x for every (scale, zero-point) the chain can produce -
-    // also for scale 0 (x / 0 is -inf, NaN, +inf in that order and NaN maps to code 0) and
-    // for NaN statistics (every code 0) - so the search runs for every channel.
-    for (int sid = wv; sid < 32 * L; sid += kFThreads / 64) {
-        const int c = sid / L, k = sid % L + 1;
-        const float sc = s_s[c], zp = s_z[c];
-        float t = NAN;   // stays NaN if no value reaches code k
-        int lo = Keys<DT>::lo - 1, hi = Keys<DT>::hi;   // code(lo) < k (lo may be the virtual floor), answer in (lo, hi]
-        bool reach = true;
-        for (int round = 0; round < 3 && reach; ++round) {
-            const int step = (hi - lo + 63) / 64;
-            const int key = min(lo + (lane + 1) * step, hi);
-            const bool pred = quant_value<DT>(key_value<DT>(key), sc, zp, levels) >= static_cast<float>(k);
-            const unsigned long long m = __ballot(pred);
-            if (m == 0) { reach = false; break; }
-            const int f = __builtin_ctzll(m);
-            hi = min(lo + (f + 1) * step, hi);
-            lo = lo + f * step;
+    // thresholds (see the statistics kernel): one 16-ary search per (channel, level) and group of
+    // 16 lanes, four rounds narrow the 2^16 ordered storage values down to one; a wave runs four
+    // searches side by side.  The code is a non-decreasing function of x for every (scale,
+    // zero-point) the chain can produce - also for scale 0 (x / 0 is -inf, NaN, +inf in that order
+    // and NaN maps to code 0) and for NaN statistics (every code 0) - so the search runs for
+    // every channel.
+    {
+        const int grp = lane >> 4, l16 = lane & 15;
+        for (int sid0 = wv * 4; sid0 < 32 * L; sid0 += kFThreads / 16) {
+            const int sid = min(sid0 + grp, 32 * L - 1);   // a group past the end repeats the last search
+            const int c = sid / L, k = sid % L + 1;
+            const float sc = s_s[c], zp = s_z[c];
+            int lo = Keys<DT>::lo - 1, hi = Keys<DT>::hi;   // code(lo) < k (lo may be the virtual floor), answer in (lo, hi]
+            bool reach = true;
+#pragma unroll
+            for (int round = 0; round < 4; ++round) {
+                const int step = (hi - lo + 15) / 16;
+                const int key = min(lo + (l16 + 1) * step, hi);
+                const bool pred = quant_value<DT>(key_value<DT>(key), sc, zp, levels) >= static_cast<float>(k);
+                const unsigned long long m = __ballot(pred);
+                const uint32_t mg = static_cast<uint32_t>(m >> (16 * grp)) & 0xffffu;   // the group's lanes
+                reach = reach && mg != 0;
+                const int f = mg ? __builtin_ctz(mg) : 0;
+                hi = min(lo + (f + 1) * step, hi);
+                lo = lo + f * step;
+            }
+            // stays NaN if no value reaches code k
+            if (l16 == 0 && sid0 + grp < 32 * L) s_thr[k - 1][c] = reach ? key_value<DT>(hi) : NAN;
         }
-        if (reach) t = key_value<DT>(hi);
-        if (lane == 0) s_thr[k - 1][c] = t;
     }
     __syncthreads();
     float th[L][8];
