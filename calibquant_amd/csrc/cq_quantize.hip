@@ -283,7 +283,8 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
                                                               uint8_t* __restrict__ codes) {
     constexpr int L = (1 << BITS) - 1;
     constexpr float levels = static_cast<float>(L);
-    __shared__ float part[kFThreads / 16][4][16];   // [wave * 4 + row of 16 lanes][piece][min x8, max x8]
+    __shared__ __attribute__((aligned(16))) float part_mn[32][kFThreads / 16];   // [channel][wave * 4 + row of 16 lanes]
+    __shared__ __attribute__((aligned(16))) float part_mx[32][kFThreads / 16];
     __shared__ float s_s[32], s_z[32], s_thr[3][32];
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int q4 = tid & 3, row = tid >> 2;
@@ -338,29 +339,33 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
         mx[j] = fmaxf(mx[j], dpp_move<0x128>(mx[j], -INFINITY));
     }
     if ((lane & 15) < 4) {
-        float* o = part[wv * 4 + (lane >> 4)][q4];
+        const int p = wv * 4 + (lane >> 4);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) { o[j] = mn[j]; o[8 + j] = mx[j]; }
+        for (int j = 0; j < 8; ++j) { part_mn[q4 * 8 + j][p] = mn[j]; part_mx[q4 * 8 + j][p] = mx[j]; }
     }
     __syncthreads();
-    if (tid < 32 && live) {   // channel c of the quarter: fold the 64 partials, run the statistics chain
-        const int c = tid;
-        float a = INFINITY, z = -INFINITY;
-#pragma unroll 4
-        for (int p = 0; p < kFThreads / 16; ++p) {
-            a = fminf(a, part[p][c >> 3][c & 7]);
-            z = fmaxf(z, part[p][c >> 3][8 + (c & 7)]);
+    // channel c of the quarter: 16 lanes fold its 64 partials (four each, then across the row),
+    // the first of them runs the statistics chain
+    if (tid < 32 * 16) {
+        const int c = tid >> 4, p16 = tid & 15;
+        const float4 a4 = *reinterpret_cast<const float4*>(&part_mn[c][4 * p16]);
+        const float4 z4 = *reinterpret_cast<const float4*>(&part_mx[c][4 * p16]);
+        float a = fminf(fminf(a4.x, a4.y), fminf(a4.z, a4.w));
+        float z = fmaxf(fmaxf(z4.x, z4.y), fmaxf(z4.z, z4.w));
+        a = row_reduce(a, OpMin(), INFINITY);
+        z = row_reduce(z, OpMax(), -INFINITY);
+        if (p16 == 0 && live) {
+            const float x_min = rnd<DT>(a * clip);
+            const float x_max = rnd<DT>(z * clip);
+            const float diff = rnd<DT>(x_max - x_min);
+            const float sc = rnd<DT>(diff * __fdiv_rn(1.0f, levels));
+            const float zp = rnd<DT>(__fdiv_rn(-x_min, sc));
+            const int64_t o = bh * g.D + quarter * 32 + c;
+            scale[o] = static_cast<uint16_t>(Cvt<DT>::from_float(sc));
+            zero[o] = static_cast<uint16_t>(Cvt<DT>::from_float(zp));
+            s_s[c] = sc;
+            s_z[c] = zp;
         }
-        const float x_min = rnd<DT>(a * clip);
-        const float x_max = rnd<DT>(z * clip);
-        const float diff = rnd<DT>(x_max - x_min);
-        const float sc = rnd<DT>(diff * __fdiv_rn(1.0f, levels));
-        const float zp = rnd<DT>(__fdiv_rn(-x_min, sc));
-        const int64_t o = bh * g.D + quarter * 32 + c;
-        scale[o] = static_cast<uint16_t>(Cvt<DT>::from_float(sc));
-        zero[o] = static_cast<uint16_t>(Cvt<DT>::from_float(zp));
-        s_s[c] = sc;
-        s_z[c] = zp;
     }
     __syncthreads();
     // thresholds (see the statistics kernel): one 16-ary search per (channel, level) and group of
