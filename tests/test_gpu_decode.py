@@ -156,6 +156,36 @@ def test_decode_attn_long_context_auto_split(ops):
     _check(_run(ops, c, "bf16", 0, 1), _oracle(c, 0, 1))
 
 
+def _sweep_cases(n, seed):
+    """Seeded draws over the options that select a code path: grouping (1 / 2 / 4 / 6 query heads per
+    kv head), token counts either side of the chunking thresholds, window lengths either side of the
+    128-row tile, dtype, bits, mask, calibration, forced chunk counts."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(n):
+        Hkv = int(rng.choice([1, 2, 8]))
+        G = int(rng.choice([1, 2, 4, 6]))
+        T = int(rng.choice([5, 63, 64, 300, 1023, 2047, 2049, 4097, 6000]))
+        B = 1 if Hkv * T > 20000 else int(rng.integers(1, 4))
+        R = int(rng.choice([0, 1, 7, 128, 129, 200, 300]))
+        S = int(rng.integers(0, min(R, 41) + 1))
+        out.append((i, B, Hkv * G, Hkv, T, R, S, int(rng.integers(1, 3)), str(rng.choice(["bf16", "fp16"])),
+                    bool(rng.random() < 0.3), bool(rng.random() < 0.8),
+                    int(rng.choice([0, 0, 2, 3])) if T >= 300 else 0))
+    return out
+
+
+@pytest.mark.parametrize("case", _sweep_cases(24, seed=5), ids=lambda c: "-".join(str(x) for x in c[1:]))
+def test_decode_attn_seeded_option_sweep(ops, case):
+    i, B, Hq, Hkv, T, R, S, bits, dtype, use_mask, calibrate, splits = case
+    c = make_case(B, Hq, Hkv, 128, T, R, bits, dtype, seed=500 + i, outlier_kind="student" if i % 2 else "x10")
+    mask = None
+    if use_mask:
+        mask = np.where(np.random.default_rng(i).random((B, T + R)) < 0.15, -1e4, 0.0).astype(np.float32)
+    got = _run(ops, c, dtype, S, bits, mask=mask, calibrate=calibrate, force_splits=splits)
+    _check(got, _oracle(c, S, bits, mask=mask, calibrate_logits=calibrate))
+
+
 def test_decode_attn_degenerate_range_and_peaked_softmax(ops):
     """All packed keys identical (logit range 0) and a residual row that takes
     nearly all the probability mass."""
