@@ -24,6 +24,7 @@
 namespace cq {
 
 constexpr int kQThreads = 256;
+constexpr int kQUnroll = 4;   // rows in flight per thread in the chunked kernels
 
 struct QuantGeom {
     int B, T, H, D;
@@ -60,12 +61,19 @@ __global__ __launch_bounds__(kQThreads) void minmax_partial_kernel(const uint16_
     float mn[8], mx[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) { mn[i] = INFINITY; mx[i] = -INFINITY; }
-    for (int t = t0 + row; t < t1; t += rows_per_iter) {
-        uint4 v = *reinterpret_cast<const uint4*>(base + t * g.st);
-        float f[8];
-        unpack8<DT>(v, f);
+    // four rows in flight per thread; rows past the chunk re-read its last row (harmless for min / max)
+    for (int tb = t0 + row; tb < t1; tb += kQUnroll * rows_per_iter) {
+        uint4 v[kQUnroll];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) { mn[i] = fminf(mn[i], f[i]); mx[i] = fmaxf(mx[i], f[i]); }
+        for (int u = 0; u < kQUnroll; ++u)
+            v[u] = *reinterpret_cast<const uint4*>(base + min(tb + u * rows_per_iter, t1 - 1) * g.st);
+#pragma unroll
+        for (int u = 0; u < kQUnroll; ++u) {
+            float f[8];
+            unpack8<DT>(v[u], f);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) { mn[i] = fminf(mn[i], f[i]); mx[i] = fmaxf(mx[i], f[i]); }
+        }
     }
     __shared__ float smn[kQThreads * 8];
     __shared__ float smx[kQThreads * 8];
@@ -193,7 +201,9 @@ __global__ __launch_bounds__(kQThreads) void emit_kernel(const uint16_t* __restr
     const int rows_per_iter = kQThreads / lpr;
     const int lane = threadIdx.x % lpr;
     const int row = threadIdx.x / lpr;
-    const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    // chunks are walked in the reverse order of the min / max launch: what that launch read last is
+    // still in the memory-side cache when this one starts
+    const int c = gridDim.x - 1 - blockIdx.x, h = gridDim.y - 1 - blockIdx.y, b = gridDim.z - 1 - blockIdx.z;
     const int t0 = c * g.chunk;
     const int t1 = min(g.T, t0 + g.chunk);
     const uint16_t* base = x + b * g.sb + h * g.sh + lane * 8;
@@ -207,60 +217,103 @@ __global__ __launch_bounds__(kQThreads) void emit_kernel(const uint16_t* __restr
         unpack8<DT>(sv, s);
         unpack8<DT>(zv, zp);
     }
-    // thresholds of this lane's 8 channels; `slow`: a channel without the step-function property
-    float th[BITS == 1 ? 1 : 3][8];
+    // thresholds of this lane's 8 channels (all three levels are loaded, as vectors, whatever BITS is);
+    // `slow`: a channel without the step-function property
+    float th[3][8];
     bool slow = false;
     {
-        const float* tp = thr + bh * 3 * g.D + lane * 8;
+        const float4* tp = reinterpret_cast<const float4*>(thr + bh * 3 * g.D + lane * 8);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-#pragma unroll
-            for (int k = 0; k < (BITS == 1 ? 1 : 3); ++k) th[k][i] = tp[k * g.D + i];
-            const float t1 = tp[g.D + i];
-            slow = slow || (th[0][i] != th[0][i] && t1 == t1);
+        for (int k = 0; k < 3; ++k) {
+            const float4 a = tp[k * (g.D >> 2)], c4 = tp[k * (g.D >> 2) + 1];
+            th[k][0] = a.x; th[k][1] = a.y; th[k][2] = a.z; th[k][3] = a.w;
+            th[k][4] = c4.x; th[k][5] = c4.y; th[k][6] = c4.z; th[k][7] = c4.w;
         }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) slow = slow | ((th[0][i] != th[0][i]) & (th[1][i] == th[1][i]));
     }
     const int nb = g.D * BITS / 8;  // bytes per packed row
-    for (int t = t0 + row; t < t1; t += rows_per_iter) {
-        uint4 v = *reinterpret_cast<const uint4*>(base + t * g.st);
-        float f[8];
-        unpack8<DT>(v, f);
-        float qv[8];
-        if (!slow) {
+    // dword stores: the lanes of a quad sit in one row (16 or 32 lanes per row) and combine their bytes
+    const bool wide = !XQ && (lpr % 4) == 0 && (reinterpret_cast<uintptr_t>(codes) & 3u) == 0;
+    const int64_t step = rows_per_iter * g.st;
+    const uint16_t* rp = base + (t0 + row) * g.st;
+    const uint16_t* last = base + (t1 - 1) * g.st;   // rows past the chunk re-read its last row
+    for (int tb = t0 + row; tb < t1; tb += kQUnroll * rows_per_iter, rp += kQUnroll * step) {
+        uint4 v[kQUnroll];   // four rows in flight per thread
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                qv[i] = (f[i] >= th[0][i]) ? 1.0f : 0.0f;
-                if constexpr (BITS == 2) {
-                    qv[i] += (f[i] >= th[1][i]) ? 1.0f : 0.0f;
-                    qv[i] += (f[i] >= th[2][i]) ? 1.0f : 0.0f;
+        for (int u = 0; u < kQUnroll; ++u)
+            v[u] = *reinterpret_cast<const uint4*>(tb + u * rows_per_iter < t1 ? rp + u * step : last);
+#pragma unroll
+        for (int u = 0; u < kQUnroll; ++u) {
+            const int t = tb + u * rows_per_iter;
+            if (t >= t1) break;   // uniform over the lanes of a row
+            float f[8];
+            unpack8<DT>(v[u], f);
+            if constexpr (XQ) {
+                float qv[8];
+                if (!slow) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        qv[i] = (f[i] >= th[0][i]) ? 1.0f : 0.0f;
+                        if constexpr (BITS == 2) {
+                            qv[i] += (f[i] >= th[1][i]) ? 1.0f : 0.0f;
+                            qv[i] += (f[i] >= th[2][i]) ? 1.0f : 0.0f;
+                        }
+                        qv[i] = (f[i] != f[i]) ? f[i] : qv[i];   // a NaN input stays NaN in x_q
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) qv[i] = quant_value<DT>(f[i], s[i], zp[i], levels);
                 }
-                if constexpr (XQ) qv[i] = (f[i] != f[i]) ? f[i] : qv[i];   // a NaN input stays NaN in x_q
-            }
-        } else {
+                uint32_t w[4];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) qv[i] = quant_value<DT>(f[i], s[i], zp[i], levels);
-        }
-        if constexpr (XQ) {
-            uint32_t w[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                w[i] = Cvt<DT>::from_float(qv[2 * i]) | (Cvt<DT>::from_float(qv[2 * i + 1]) << 16);
-            uint16_t* o = xq + ((static_cast<int64_t>(b) * g.T + t) * g.H + h) * g.D + lane * 8;
-            *reinterpret_cast<uint4*>(o) = make_uint4(w[0], w[1], w[2], w[3]);
-        } else {
-            uint32_t code[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) code[i] = (qv[i] != qv[i]) ? 0u : static_cast<uint32_t>(qv[i]);
-            uint8_t* o = codes + (bh * g.T + t) * nb;
-            if constexpr (BITS == 1) {
-                uint32_t byte = 0;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) byte |= code[i] << (7 - i);
-                o[lane] = static_cast<uint8_t>(byte);
+                for (int i = 0; i < 4; ++i)
+                    w[i] = Cvt<DT>::from_float(qv[2 * i]) | (Cvt<DT>::from_float(qv[2 * i + 1]) << 16);
+                uint16_t* o = xq + ((static_cast<int64_t>(b) * g.T + t) * g.H + h) * g.D + lane * 8;
+                *reinterpret_cast<uint4*>(o) = make_uint4(w[0], w[1], w[2], w[3]);
             } else {
-                uint32_t b0 = (code[0] << 6) | (code[1] << 4) | (code[2] << 2) | code[3];
-                uint32_t b1 = (code[4] << 6) | (code[5] << 4) | (code[6] << 2) | code[7];
-                reinterpret_cast<uint16_t*>(o)[lane] = static_cast<uint16_t>(b0 | (b1 << 8));
+                uint32_t code[8];
+                if (!slow) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {   // a NaN input compares false: code 0
+                        code[i] = (f[i] >= th[0][i]) ? 1u : 0u;
+                        if constexpr (BITS == 2) {
+                            code[i] += (f[i] >= th[1][i]) ? 1u : 0u;
+                            code[i] += (f[i] >= th[2][i]) ? 1u : 0u;
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        const float qv = quant_value<DT>(f[i], s[i], zp[i], levels);
+                        code[i] = (qv != qv) ? 0u : static_cast<uint32_t>(qv);
+                    }
+                }
+                uint8_t* o = codes + (bh * g.T + t) * nb;
+                if constexpr (BITS == 1) {
+                    uint32_t byte = 0;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) byte |= code[i] << (7 - i);
+                    if (wide) {
+                        int w = static_cast<int>(byte << (8 * (lane & 3)));
+                        w |= dpp_move_i<0xB1>(w, 0);
+                        w |= dpp_move_i<0x4E>(w, 0);
+                        if ((lane & 3) == 0) *reinterpret_cast<uint32_t*>(o + lane) = static_cast<uint32_t>(w);
+                    } else {
+                        o[lane] = static_cast<uint8_t>(byte);
+                    }
+                } else {
+                    const uint32_t b0 = (code[0] << 6) | (code[1] << 4) | (code[2] << 2) | code[3];
+                    const uint32_t b1 = (code[4] << 6) | (code[5] << 4) | (code[6] << 2) | code[7];
+                    const uint32_t half = b0 | (b1 << 8);
+                    if (wide) {
+                        int w = static_cast<int>(half << (16 * (lane & 1)));
+                        w |= dpp_move_i<0xB1>(w, 0);
+                        if ((lane & 1) == 0) *reinterpret_cast<uint32_t*>(o + 2 * lane) = static_cast<uint32_t>(w);
+                    } else {
+                        reinterpret_cast<uint16_t*>(o)[lane] = static_cast<uint16_t>(half);
+                    }
+                }
             }
         }
     }
