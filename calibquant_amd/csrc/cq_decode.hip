@@ -38,11 +38,9 @@
 namespace cq {
 
 constexpr int kD = 128;
-constexpr int kNT = 1024;          // threads per workgroup
-constexpr int kNW = kNT / kWave;   // waves per workgroup
 constexpr int kPF = 4;             // 16-byte loads kept in flight per thread and stream
-constexpr int kResTile = kNT / 8;  // residual rows per tile (8 lanes per row)
 constexpr int kLdsMax = 160 * 1024;
+constexpr int kPairUnits = 256;    // compute units of the device this is laid out for
 constexpr float kLog2e = 1.4426950408889634f;
 
 template <int N> struct alignas(N * 4) Vec { float v[N]; };
@@ -79,7 +77,13 @@ constexpr int cmin(int a, int b) { return a < b ? a : b; }
 // codes in little-endian 32-bit words, first channel in the lowest bits) instead of per
 // channel.  A token slot then also carries the token's group scales, and every channel
 // group has its own subset-sum tables.
-template <int BITS, int HPB, bool VTOK = false> struct Lay {
+// F16K: the K table entries, the look-up sums and the logits waiting in the token slots are packed
+// fp16 (half the LDS bytes, so that two 512-thread workgroups fit a compute unit's LDS); the
+// reference's own look-up kernel stores its logits as fp16 as well (calibquant.py:104-111).
+template <int BITS, int HPB, bool VTOK = false, int NT_ = 1024, bool F16K = false> struct Lay {
+    static constexpr int kNT = NT_;                 // threads per workgroup
+    static constexpr int kNW = kNT / kWave;         // waves per workgroup
+    static constexpr int kResTile = kNT / 8;        // residual rows per tile (8 lanes per row)
     static constexpr int NB = 16 * BITS;            // bytes per packed row
     static constexpr int PC = NB * 8;               // bit lanes per row
     static constexpr int GPW = kWave / NB;          // 4-token groups per wave pass
@@ -91,12 +95,14 @@ template <int BITS, int HPB, bool VTOK = false> struct Lay {
     // The byte-indexed K table covers NBP byte positions at a time: all of them when that fits
     // 64 KB, else half of them in each of two passes over the chunk's rows (one 16-byte piece
     // of a 2-bit row per pass), the first pass's partial logits waiting in the token slots.
-    static constexpr int KPASS = (NB * 256 * ESZ > 64 * 1024) ? 2 : 1;
+    static constexpr int KESZ = F16K ? ESZH : ESZ;  // bytes per K table entry and per waiting logits slot
+    static constexpr int KPASS = (NB * 256 * KESZ > 64 * 1024) ? 2 : 1;
     static constexpr int NBP = NB / KPASS;          // byte positions per pass
     static constexpr int PPP = BITS / KPASS;        // 16-byte pieces of a row per pass
-    static constexpr int KT = NBP * 256 * ESZ;      // K table bytes
+    static constexpr int KT = NBP * 256 * KESZ;     // K table bytes
+    static_assert(!F16K || (KPASS == 1 && !VTOK && HPB >= 2), "packed-fp16 logits: one table pass, per-channel values");
     static_assert(KPASS == 1 || (KPASS == 2 && BITS == 2), "a pass consumes whole 16-byte pieces");
-    static constexpr int SLOT = VTOK ? 16 : ESZ;    // bytes per token slot: logits, later e (+ 4 group scales)
+    static constexpr int SLOT = VTOK ? 16 : KESZ;   // bytes per token slot: logits, later e (+ 4 group scales)
     static constexpr int NGRP = VTOK ? kD / 32 : 1; // channel groups with tables of their own
     static constexpr int WTAB = kNW * NGRP * GPW * 16 * ESZH;
     static constexpr int RW = cmax(3 * HPB, VTOK ? (NGRP + 1) * HPB : 0);   // per-wave partials: min/max + masked max, or the closing sums
@@ -113,14 +119,16 @@ template <int BITS, int HPB, bool VTOK = false> struct Lay {
     static constexpr int F_STAT = F_RED + kNW * RW;           // 8*HPB: per-head softmax state
     static constexpr int F_VSZ = F_STAT + 8 * HPB;            // 2*kD: value scale, zero-point (VTOK: NGRP*HPB minimum terms)
     static constexpr int F_NIB = F_VSZ + 2 * kD;              // NB*32*HPB: nibble tables
-    static constexpr int F_SRES = F_NIB + NB * 32 * HPB;      // kResTile*HPB
+    // (F16K: the nibble tables live in the token slots, which are first written after the table build)
+    static constexpr int NIBF = NB * 32 * HPB;
+    static constexpr int F_SRES = F_NIB + (F16K ? 0 : NIBF);  // kResTile*HPB
     static constexpr int F_PRES = F_SRES + kResTile * HPB;    // kResTile*HPB
     static constexpr int F_END = F_PRES + kResTile * HPB;
     static constexpr int FIXED = ((F_END * 4 + 255) / 256) * 256;
     static constexpr int region_a(int cap) {
         return (cmax(cmax(KT, WTAB + cmin(VSUB, cap) * NB), cmax(RED, RED2)) + 255) / 256 * 256;
     }
-    static constexpr int lds_bytes(int cap) { return region_a(cap) + FIXED + cap * SLOT; }
+    static constexpr int lds_bytes(int cap) { return region_a(cap) + FIXED + cmax(cap * SLOT, F16K ? NIBF * 4 : 0); }
     static constexpr int max_chunk() {
         int best = 64;
         for (int c = 64; c <= 16384; c += 64)
@@ -143,7 +151,7 @@ __device__ __forceinline__ void max_step(int* k) {
 
 // Block-wide maximum of N values (integer keys, see float_key); result wave-uniform.
 // One barrier; `red` (kNW * N words) must not be rewritten before the next barrier of the caller.
-template <int N>
+template <int N, int kNW>
 __device__ __forceinline__ void block_max(float* v, float* red) {
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     int* redi = reinterpret_cast<int*>(red);
@@ -227,11 +235,12 @@ __device__ __forceinline__ uint32_t pack_f16(float a, float b) {
     return __builtin_bit_cast(uint32_t, h);
 }
 
-template <int BITS, int HPB, typename DT, bool MINMAX_ONLY, bool VTOK = false>
-__global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
-    using L = Lay<BITS, HPB, VTOK>;
+template <int BITS, int HPB, typename DT, bool MINMAX_ONLY, bool VTOK = false, int NT = 1024, bool F16K = false>
+__global__ __launch_bounds__(NT) void decode_kernel(DecodeGeom g) {
+    using L = Lay<BITS, HPB, VTOK, NT, F16K>;
     using V = Vec<HPB>;
     constexpr int NB = L::NB;
+    constexpr int kNT = L::kNT, kNW = L::kNW, kResTile = L::kResTile;
     extern __shared__ __attribute__((aligned(256))) unsigned char smem[];
     const int reg_a = L::region_a(g.cap);
     unsigned char* regA = smem;
@@ -276,15 +285,23 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
     // at q (always mapped, at least 256 bytes) and never looks at what comes back.
     const bool has_img = n > 0;
     uint32_t q_raw, s_raw, z_raw;
+    constexpr bool kVSep = (HPB * kD > kNT - kD);
+    uint32_t vs_raw = 0, vz_raw = 0;
     {
         const int h = min(tid / kD, HPB - 1), d = tid % kD;
         const uint16_t* qp = static_cast<const uint16_t*>(g.q) + (static_cast<int64_t>(b) * g.Hq + hq0) * kD;
         q_raw = qp[h * kD + d];
-        const bool vstat = tid >= kNT - kD;   // the last kD threads fetch the value statistics
+        // the last kD threads fetch the value statistics, unless they are q threads as well
+        // (then the first kD threads fetch them with two loads of their own, below)
+        const bool vstat = tid >= kNT - kD && !kVSep;
         const uint16_t* sp = has_img ? static_cast<const uint16_t*>((vstat && !VTOK) ? g.vs : g.ks) + bh * kD : qp;
         const uint16_t* zp = has_img ? static_cast<const uint16_t*>((vstat && !VTOK) ? g.vz : g.kz) + bh * kD : qp;
         s_raw = sp[d];
         z_raw = zp[d];
+        if constexpr (kVSep && !VTOK) {
+            vs_raw = (has_img ? static_cast<const uint16_t*>(g.vs) + bh * kD : qp)[d];
+            vz_raw = (has_img ? static_cast<const uint16_t*>(g.vz) + bh * kD : qp)[d];
+        }
     }
     const int64_t code_off = has_img ? (bh * g.T + t0) * NB : 0;   // one offset for both code streams
     const uint4* ckp = reinterpret_cast<const uint4*>((has_img ? g.ck : static_cast<const uint8_t*>(g.q)) + code_off);
@@ -340,7 +357,12 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
             }
         }
     }
-    if (!VTOK && n > 0 && tid >= kNT - kD && tid >= HPB * kD) {
+    if constexpr (kVSep) {
+        if (!VTOK && n > 0 && tid < kD) {
+            fx[L::F_VSZ + tid] = Cvt<DT>::to_float(vs_raw);
+            fx[L::F_VSZ + kD + tid] = Cvt<DT>::to_float(vz_raw);
+        }
+    } else if (!VTOK && n > 0 && tid >= kNT - kD) {
         const int d = tid - (kNT - kD);
         fx[L::F_VSZ + d] = Cvt<DT>::to_float(s_raw);
         fx[L::F_VSZ + kD + d] = Cvt<DT>::to_float(z_raw);
@@ -361,6 +383,39 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
     float mn[HPB], mx[HPB];
 #pragma unroll
     for (int h = 0; h < HPB; ++h) { mn[h] = INFINITY; mx[h] = -INFINITY; }
+    // F16K: running min / max of the packed logits, two heads per register
+    f16x2_t mnp[L::HW], mxp[L::HW];
+#pragma unroll
+    for (int k = 0; k < L::HW; ++k) {
+        mnp[k] = f16x2_t{static_cast<_Float16>(INFINITY), static_cast<_Float16>(INFINITY)};
+        mxp[k] = f16x2_t{static_cast<_Float16>(-INFINITY), static_cast<_Float16>(-INFINITY)};
+    }
+    using KW = Words<L::HW>;   // a packed-fp16 entry: the unit's heads, two per word
+    // logits (later: calibrated, masked logits) waiting in a token's slot
+    auto load_logits = [&](int tt) {
+        V w;
+        if constexpr (F16K) {
+            const KW r = *reinterpret_cast<const KW*>(slot(tt));
+#pragma unroll
+            for (int h = 0; h < HPB; ++h) {
+                const f16x2_t pr = __builtin_bit_cast(f16x2_t, r.w[h >> 1]);
+                w.v[h] = static_cast<float>((h & 1) ? pr.y : pr.x);
+            }
+        } else {
+            w = *reinterpret_cast<const V*>(slot(tt));
+        }
+        return w;
+    };
+    auto store_logits = [&](int tt, const V& w) {
+        if constexpr (F16K) {
+            KW r;
+#pragma unroll
+            for (int k = 0; k < L::HW; ++k) r.w[k] = pack_f16(w.v[2 * k], w.v[2 * k + 1]);
+            *reinterpret_cast<KW*>(slot(tt)) = r;
+        } else {
+            *reinterpret_cast<V*>(slot(tt)) = w;
+        }
+    };
     // First block of packed V rows: half of it is requested here, behind the packed K rows, the
     // rest as the K registers free up, so it has arrived when the logits are done.
     U4 vc[kPF];
@@ -375,7 +430,7 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
         // ---- phase 2: byte table = high-nibble table + low-nibble table ----------------
         // nibble tables: entry (j, half, v) = sum of the per-bit weights v selects; the
         // zero-point sum of the byte position is folded into the high half.
-        V* nib = reinterpret_cast<V*>(fx + L::F_NIB);   // [half*16 + value][byte position]
+        V* nib = F16K ? reinterpret_cast<V*>(slots) : reinterpret_cast<V*>(fx + L::F_NIB);   // [half*16 + value][byte position]
         V* ktab = reinterpret_cast<V*>(regA);           // [byte value][byte position]
         for (int e = tid; e < NB * 32; e += kNT) {
             const int j = e % NB, half = (e / NB) >> 4, v = (e / NB) & 15;
@@ -411,12 +466,12 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
         const uint32_t bsel = (0x03020100u ^ (0x01010101u * (skew & 3)));
         uint32_t pofs[NBP];   // byte offset of position k ^ skew inside a table row
 #pragma unroll
-        for (int k = 0; k < NBP; ++k) pofs[k] = (k ^ skew) * L::ESZ;
+        for (int k = 0; k < NBP; ++k) pofs[k] = (k ^ skew) * L::KESZ;
         const unsigned char* ktab_b = regA;
         // With 256-byte table rows the address of a look-up is two bytes side by side, the
         // byte value above the position offset: one byte permute builds it from the row word
         // and a word holding four position offsets.
-        constexpr bool kPermAddr = (NBP * L::ESZ == 256);
+        constexpr bool kPermAddr = (NBP * L::KESZ == 256) && !F16K;
         uint32_t pofs4[NBP / 4];
 #pragma unroll
         for (int i = 0; i < NBP / 4; ++i)
@@ -444,6 +499,42 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
 #pragma unroll
                 for (int i = 0; i < NW32; ++i) wds[i] = __builtin_amdgcn_perm(w[i], w[i], bsel);
                 // balanced-tree sum with a small stack of partial sums (level l holds 2^l terms)
+                if constexpr (F16K) {
+                    f16x2_t part[6][L::HW];
+#pragma unroll
+                    for (int k = 0; k < NBP; ++k) {
+                        // absolute LDS address (the table starts at 0): table row of the byte value, position inside
+                        const uint32_t byte = (wds[k >> 2] >> (8 * (k & 3))) & 0xffu;
+                        const KW r = lds_words<L::HW>(byte * (NBP * L::KESZ) + pofs[k]);
+                        f16x2_t cur[L::HW];
+#pragma unroll
+                        for (int i = 0; i < L::HW; ++i) cur[i] = __builtin_bit_cast(f16x2_t, r.w[i]);
+#pragma unroll
+                        for (int l = 0; l < 6; ++l) {
+                            if ((k >> l) & 1) {
+#pragma unroll
+                                for (int i = 0; i < L::HW; ++i) cur[i] += part[l][i];
+                            } else {
+#pragma unroll
+                                for (int i = 0; i < L::HW; ++i) part[l][i] = cur[i];
+                                break;
+                            }
+                        }
+                        if (k == NBP - 1) {
+#pragma unroll
+                            for (int i = 0; i < L::HW; ++i) part[5][i] = cur[i];
+                        }
+                        if ((k & 7) == 7) __builtin_amdgcn_sched_barrier(0);
+                    }
+                    KW o;
+#pragma unroll
+                    for (int i = 0; i < L::HW; ++i) {
+                        o.w[i] = __builtin_bit_cast(uint32_t, part[5][i]);
+                        mnp[i] = __builtin_elementwise_min(mnp[i], part[5][i]);
+                        mxp[i] = __builtin_elementwise_max(mxp[i], part[5][i]);
+                    }
+                    *reinterpret_cast<KW*>(slot(tt)) = o;
+                } else {
                 V part[6];
 #pragma unroll
                 for (int k = 0; k < NBP; ++k) {
@@ -483,6 +574,7 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
 #pragma unroll
                     for (int h = 0; h < HPB; ++h) { mn[h] = fminf(mn[h], acc.v[h]); mx[h] = fmaxf(mx[h], acc.v[h]); }
                 }
+                }
             }
         };
         auto k_pass = [&](auto pass_c) {
@@ -495,7 +587,14 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                 V o;
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) o.v[h] = hi.v[h] + lo.v[h];
-                ktab[e] = o;
+                if constexpr (F16K) {
+                    KW o16;
+#pragma unroll
+                    for (int i = 0; i < L::HW; ++i) o16.w[i] = pack_f16(o.v[2 * i], o.v[2 * i + 1]);
+                    reinterpret_cast<KW*>(regA)[e] = o16;
+                } else {
+                    ktab[e] = o;
+                }
             }
             __syncthreads();
             // first batch: rows already in registers; each consumed round of the last pass frees
@@ -533,11 +632,18 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
             k_pass(std::integral_constant<int, 1>{});
         }
     }
+    if constexpr (F16K) {
+#pragma unroll
+        for (int h = 0; h < HPB; ++h) {
+            mn[h] = static_cast<float>((h & 1) ? mnp[h >> 1].y : mnp[h >> 1].x);
+            mx[h] = static_cast<float>((h & 1) ? mxp[h >> 1].y : mxp[h >> 1].x);
+        }
+    }
     if (n > 0) {   // one reduction for both: max of (-min, max)
         float mm2[2 * HPB];
 #pragma unroll
         for (int h = 0; h < HPB; ++h) { mm2[h] = -mn[h]; mm2[HPB + h] = mx[h]; }
-        block_max<2 * HPB>(mm2, red);
+        block_max<2 * HPB, kNW>(mm2, red);
 #pragma unroll
         for (int h = 0; h < HPB; ++h) { mn[h] = -mm2[h]; mx[h] = mm2[HPB + h]; }
     }
@@ -623,16 +729,17 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) lm[h] = -INFINITY;
                 for (int tt = tid; tt < n; tt += kNT) {
-                    V w = *reinterpret_cast<const V*>(slot(tt));
+                    V w = load_logits(tt);
                     const float mv = mk[tt];
 #pragma unroll
                     for (int h = 0; h < HPB; ++h) {
                         w.v[h] = (w.v[h] - mn[h]) * slope[h] + tmin[h] + mv;
+                        if constexpr (F16K) w.v[h] = static_cast<float>(static_cast<_Float16>(w.v[h]));   // as it will wait in the slot
                         lm[h] = fmaxf(lm[h], w.v[h]);
                     }
-                    *reinterpret_cast<V*>(slot(tt)) = w;
+                    store_logits(tt, w);
                 }
-                block_max<HPB>(lm, red + kNW * 2 * HPB);   // the first reduction's words may still be read
+                block_max<HPB, kNW>(lm, red + kNW * 2 * HPB);   // the first reduction's words may still be read
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) { m_img[h] = lm[h]; slope[h] = 1.0f; tmin[h] = 0.f; mn[h] = 0.f; }
             } else {
@@ -661,7 +768,7 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                 float e[4] = {0.f, 0.f, 0.f, 0.f};
                 uint32_t sc2[2] = {0u, 0u};   // the token's group scales as fp16
                 if (tt < n) {
-                    const V w = *reinterpret_cast<const V*>(slot(tt));
+                    const V w = load_logits(tt);
 #pragma unroll
                     for (int h = 0; h < HPB; ++h) {
                         // (w - mn) first: with a degenerate logit range the slope is ~1e8 and only the exact
@@ -935,17 +1042,25 @@ __global__ __launch_bounds__(kNT) void decode_kernel(DecodeGeom g) {
                 __syncthreads();
                 if (wv < HPB) {   // wave h keeps the running softmax state of head h
                     const int h = wv;
-                    const float s0 = sres[lane * HPB + h];
-                    const float s1 = sres[(lane + 64) * HPB + h];
-                    const float mnew = fmaxf(m_run, wave_max(fmaxf(s0, s1)));
+                    constexpr int kRL = kResTile / kWave;   // tile rows per lane
+                    float sv[kRL], smax = -INFINITY;
+#pragma unroll
+                    for (int i = 0; i < kRL; ++i) {
+                        sv[i] = sres[(lane + i * kWave) * HPB + h];
+                        smax = fmaxf(smax, sv[i]);
+                    }
+                    const float mnew = fmaxf(m_run, wave_max(smax));
                     const bool dead = (mnew == -INFINITY);
-                    const float p0 = dead ? 0.f : __expf(s0 - mnew);
-                    const float p1 = dead ? 0.f : __expf(s1 - mnew);
+                    float psum = 0.f;
+#pragma unroll
+                    for (int i = 0; i < kRL; ++i) {
+                        const float pi = dead ? 0.f : __expf(sv[i] - mnew);
+                        pres[(lane + i * kWave) * HPB + h] = pi;
+                        psum += pi;
+                    }
                     const float al = dead ? 1.0f : __expf(m_run - mnew);
-                    l_run = l_run * al + wave_sum(p0 + p1);
+                    l_run = l_run * al + wave_sum(psum);
                     m_run = mnew;
-                    pres[lane * HPB + h] = p0;
-                    pres[(lane + 64) * HPB + h] = p1;
                     if (lane == 0) { stat[h] = al; stat[HPB + h] = m_run; stat[2 * HPB + h] = l_run; }
                 }
                 __syncthreads();
@@ -1035,13 +1150,13 @@ __global__ void merge_kernel(const float* __restrict__ part, int nx, void* __res
 }
 
 struct Plan {
-    int hpb, nsplit, chunk, nx, cap, lds;
+    int hpb, nt, nsplit, chunk, nx, cap, lds;
     size_t ws_mm, ws_part;
 };
 
-template <int BITS, int HPB, bool VTOK>
+template <int BITS, int HPB, bool VTOK, int NT = 1024, bool F16K = false>
 static void plan_for(const cq_decode_args* a, Plan* p) {
-    using L = Lay<BITS, HPB, VTOK>;
+    using L = Lay<BITS, HPB, VTOK, NT, F16K>;
     const int G = a->Hq / a->Hkv;
     const int64_t units = static_cast<int64_t>(a->B) * a->Hkv * (G / HPB);
     const int maxc = L::max_chunk();
@@ -1062,6 +1177,7 @@ static void plan_for(const cq_decode_args* a, Plan* p) {
     if (chunk > maxc) chunk = maxc;
     nsplit = a->T > 0 ? (a->T + chunk - 1) / chunk : 1;
     p->hpb = HPB;
+    p->nt = NT;
     p->nsplit = nsplit;
     p->chunk = chunk;
     p->nx = nsplit + ((nsplit > 1 && a->R > 0) ? 1 : 0);
@@ -1087,6 +1203,15 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
         if (G % 4 == 0) vtok ? plan_for<1, 4, true>(a, p) : plan_for<1, 4, false>(a, p);
         else if (G % 2 == 0) vtok ? plan_for<1, 2, true>(a, p) : plan_for<1, 2, false>(a, p);
         else vtok ? plan_for<1, 1, true>(a, p) : plan_for<1, 1, false>(a, p);
+        // More units than compute units: 512-thread workgroups, two resident per compute unit, keep its
+        // pipes busier than one 1024-thread workgroup after the other (one unit's LDS-bound and
+        // barrier-bound phases overlap the other's arithmetic) - when a unit's whole layout fits half the LDS.
+        const int64_t units = static_cast<int64_t>(a->B) * a->Hkv * (G / p->hpb);
+        if (!vtok && a->force_splits == 0 && p->nsplit == 1 && units > kPairUnits && p->hpb >= 2) {
+            Plan q;
+            if (p->hpb == 4) plan_for<1, 4, false, 512, true>(a, &q); else plan_for<1, 2, false, 512, false>(a, &q);
+            if (q.nsplit == 1 && q.lds <= kLdsMax / 2) *p = q;
+        }
     } else {
         // four heads per unit need the two-pass K table; with per-token values their LDS layout
         // would not hold a 3 328-token chunk, so that mode keeps two heads per unit
@@ -1099,12 +1224,13 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
     return CQ_OK;
 }
 
-template <int BITS, int HPB, typename DT, bool VTOK>
+template <int BITS, int HPB, typename DT, bool VTOK, int NT = 1024, bool F16K = false>
 static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
     const int G = g.Hq / g.Hkv;
     const unsigned units = static_cast<unsigned>(g.B) * g.Hkv * (G / HPB);
-    auto kmain = decode_kernel<BITS, HPB, DT, false, VTOK>;
-    auto kmm = decode_kernel<BITS, HPB, DT, true, false>;   // the min/max pass never looks at values
+    auto kmain = decode_kernel<BITS, HPB, DT, false, VTOK, NT, F16K>;
+    // the min/max pass never looks at values (the 512-thread plans are single-launch: it is never run for them)
+    auto kmm = decode_kernel<BITS, HPB, DT, true, false, 1024, false>;
     // raise the dynamic-LDS limit once per device for this instantiation
     static std::atomic<uint32_t> attr_done{0};
     int dev = 0;
@@ -1133,12 +1259,13 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
         g1.nx = g.nsplit;  // the min/max pass has no residual unit
         g1.d_nx.set(static_cast<uint32_t>(g.nsplit));
         // ... and keeps no logits, unless the table takes two passes (partial logits wait in the slots)
+        if (NT != 1024) return CQ_ERR_UNSUPPORTED;
         g1.cap = Lay<BITS, HPB, false>::KPASS > 1 ? p.cap : 0;
         const int lds_mm = Lay<BITS, HPB, false>::lds_bytes(g1.cap);
-        hipLaunchKernelGGL(kmm, dim3(units * g.nsplit), dim3(kNT), lds_mm, st, g1);
+        hipLaunchKernelGGL(kmm, dim3(units * g.nsplit), dim3(1024), lds_mm, st, g1);
         CQ_LAUNCH_CHECK();
     }
-    hipLaunchKernelGGL(kmain, dim3(units * g.nx), dim3(kNT), p.lds, st, gm);
+    hipLaunchKernelGGL(kmain, dim3(units * g.nx), dim3(NT), p.lds, st, gm);
     CQ_LAUNCH_CHECK();
     if (g.nsplit > 1) {
         hipLaunchKernelGGL(merge_kernel<DT>, dim3(static_cast<unsigned>(g.B) * g.Hq), dim3(kD), 0, st, g.part, g.nx,
@@ -1151,6 +1278,10 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
 template <typename DT, bool VTOK>
 static int dispatch(const DecodeGeom& g, const Plan& p, int bits, hipStream_t st) {
     if (bits == 1) {
+        if constexpr (!VTOK) {
+            if (p.hpb == 4 && p.nt == 512) return launch<1, 4, DT, false, 512, true>(g, p, st);
+            if (p.hpb == 2 && p.nt == 512) return launch<1, 2, DT, false, 512, false>(g, p, st);
+        }
         if (p.hpb == 4) return launch<1, 4, DT, VTOK>(g, p, st);
         if (p.hpb == 2) return launch<1, 2, DT, VTOK>(g, p, st);
         return launch<1, 1, DT, VTOK>(g, p, st);

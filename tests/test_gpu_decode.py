@@ -211,6 +211,67 @@ def test_decode_attn_full_batch_properties(ops):
     _check(to_np(out[:2]), _oracle(c, 0, 1))
 
 
+PAIRED = [
+    # reps, Hq, Hkv, T, R, S, dtype, mask, calibrate — more than 256 units of work, a unit's layout within half the LDS:
+    # the launch uses 512-thread workgroups, two per compute unit (four heads per unit: packed-fp16 logits)
+    (20, 32, 8, 777, 60, 41, "bf16", False, True),
+    (20, 32, 8, 3328, 128, 0, "fp16", False, True),
+    (20, 32, 8, 2100, 70, 5, "bf16", True, True),       # two blocks of staged value rows, mask
+    (20, 32, 8, 300, 0, 0, "fp16", False, False),
+    (20, 16, 8, 1500, 130, 3, "bf16", True, True),      # two heads per unit: fp32 logits
+    (17, 48, 8, 1000, 33, 0, "fp16", False, True),      # six q heads per kv head: three units of two heads
+    (20, 32, 8, 0, 200, 0, "bf16", False, True),        # window only
+]
+
+
+@pytest.mark.parametrize("case", PAIRED, ids=lambda c: "-".join(str(x) for x in c))
+def test_decode_attn_paired_workgroups(ops, case):
+    """Batches with more units of work than compute units: every batch row is an independent problem, so
+    a two-row case repeated `reps` times gives identical outputs per repetition, and the first two
+    rows equal the oracle."""
+    reps, Hq, Hkv, T, R, S, dtype, use_mask, calibrate = case
+    c = make_case(2, Hq, Hkv, 128, max(T, 1), R, 1, dtype, seed=60 + T, outlier_kind="x10" if T % 2 else "student")
+    if T == 0:
+        c["ck"], c["cv"] = c["ck"][:, :, :0], c["cv"][:, :, :0]
+    mask = None
+    if use_mask:
+        mask = np.where(np.random.default_rng(T).random((2, T + R)) < 0.15, -1e4, 0.0).astype(np.float32)
+    g = case_to_gpu(c, dtype)
+    rep = {k: torch.cat([v] * reps, 0) for k, v in g.items()}
+    m = None if mask is None else torch.from_numpy(mask).cuda().repeat(reps, 1)
+    args = [rep[k] if T else None for k in ("ck", "cv", "sk", "zk", "sv", "zv")]
+    out = ops.decode_attn(rep["q"], *args, rep["kr"] if R else None, rep["vr"] if R else None,
+                          sprompt_len=S, bits=1, mask=m, calibrate=calibrate)
+    torch.cuda.synchronize()
+    assert torch.equal(out, out[:2].repeat(reps, 1, 1))
+    _check(to_np(out[:2]), _oracle(c, S, 1, mask=mask, calibrate_logits=calibrate))
+
+
+def test_decode_attn_paired_workgroups_row_count_on_device(ops):
+    """The 512-thread launch with the window's row count in a device scalar (a recorded decode step at a
+    large batch)."""
+    reps, Hq, Hkv, T, R, S = 20, 32, 8, 1500, 150, 41
+    c = make_case(2, Hq, Hkv, 128, T, R, 1, "bf16", seed=23)
+    g = case_to_gpu(c, "bf16")
+    rep = {k: torch.cat([v] * reps, 0) for k, v in g.items()}
+    cap = 192
+    kbuf = torch.full((2 * reps, Hkv, cap, 128), 1e4, dtype=torch.bfloat16, device="cuda")
+    vbuf = torch.full_like(kbuf, -1e4)
+    kbuf[:, :, :R] = rep["kr"]
+    vbuf[:, :, :R] = rep["vr"]
+    r_dev = torch.zeros(1, dtype=torch.int32, device="cuda")
+    call = ops.DecodeCall(rep["q"], rep["ck"], rep["cv"], rep["sk"], rep["zk"], rep["sv"], rep["zv"], kbuf, vbuf,
+                          sprompt_len=S, bits=1, r_dev=r_dev)
+    for rows in (60, 150, 129):
+        r_dev.fill_(rows)
+        out = call.run()
+        torch.cuda.synchronize()
+        assert torch.equal(out, out[:2].repeat(reps, 1, 1))
+        want = O.decode_attention(c["q"], c["ck"], c["cv"], c["sk"], c["zk"], c["sv"], c["zv"],
+                                  c["kr"][:, :, :rows], c["vr"][:, :, :rows], S, 1)
+        _check(to_np(out[:2]), want)
+
+
 def test_decode_attn_rejects_bad_arguments(ops):
     from calibquant_amd._lib import CalibQuantError
     c = make_case(1, 32, 8, 128, 64, 8, 1, "bf16", seed=1)
