@@ -1,7 +1,9 @@
 // Fused decode attention over bit-packed K/V for gfx950 (MI355X).
 //
-// One 1024-thread workgroup owns one (batch, kv-head, head-group, token-chunk)
-// unit and runs the whole step for HPB query heads that share the kv-head:
+// One workgroup (1024 threads, or 512 threads with two workgroups resident per compute
+// unit when there are more units than compute units) owns one (batch, kv-head,
+// head-group, token-chunk) unit and runs the whole step for HPB query heads that share
+// the kv-head:
 //
 //   loads    the packed K rows are requested at kernel entry, the first block of
 //            packed V rows behind them (half before the logits, half as the K
@@ -1203,9 +1205,9 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
         if (G % 4 == 0) vtok ? plan_for<1, 4, true>(a, p) : plan_for<1, 4, false>(a, p);
         else if (G % 2 == 0) vtok ? plan_for<1, 2, true>(a, p) : plan_for<1, 2, false>(a, p);
         else vtok ? plan_for<1, 1, true>(a, p) : plan_for<1, 1, false>(a, p);
-        // More units than compute units: 512-thread workgroups, two resident per compute unit, keep its
-        // pipes busier than one 1024-thread workgroup after the other (one unit's LDS-bound and
-        // barrier-bound phases overlap the other's arithmetic) - when a unit's whole layout fits half the LDS.
+        // More units than compute units: 512-thread workgroups, two resident per compute unit, need fewer
+        // instructions per unit than one 1024-thread workgroup after the other (half as many waves pay
+        // the per-wave set-up, reductions and folds) - when a unit's whole layout fits half the LDS.
         const int64_t units = static_cast<int64_t>(a->B) * a->Hkv * (G / p->hpb);
         if (!vtok && a->force_splits == 0 && p->nsplit == 1 && units > kPairUnits && p->hpb >= 2) {
             Plan q;
