@@ -384,6 +384,7 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
     ms = time_calls(torch, calls, a.steps, a.warmup)
+    plan = calls[0].plan()
     nbytes = algorithmic_bytes(B, Hq, Hkv, D, T, R, a.bits)
     gbps = nbytes / (ms * 1e-3) / 1e9
 
@@ -398,11 +399,12 @@ def main():
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        # fp32 accumulation throughout; the paired 512-thread launch sums its K look-ups in packed fp16
+        "dtype": "f32+f16" if plan["f16_logits"] else "f32",
         "data": "synthetic",
         "config": {"workload": a.workload, "batch": B, "q_heads": Hq, "kv_heads": Hkv, "head_dim": D,
                    "kv_packed_tokens": T, "kv_residual_rows": R, "bits": a.bits, "storage_dtype": "bf16",
-                   "buffer_sets": a.sets, "launches_per_step": 1 if calls[0].workspace_bytes == 0 else 3},
+                   "buffer_sets": a.sets, "launches_per_step": plan["launches"], "launch_plan": plan},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": measured_traffic(a.workload, a.bits),
                      "algorithmic_bytes": nbytes},

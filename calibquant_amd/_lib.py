@@ -16,8 +16,14 @@ SYMBOLS = (
     "cq_version", "cq_strerror", "cq_last_hip_error",
     "cq_quantize_pack_workspace", "cq_quantize_pack", "cq_quant", "cq_encode",
     "cq_lut_vecmat_qk", "cq_lut_vecmat_pv",
-    "cq_decode_attn_workspace", "cq_decode_attn", "cq_rope_append", "cq_quantize_pack_token",
+    "cq_decode_attn_workspace", "cq_decode_attn", "cq_decode_attn_plan", "cq_rope_append", "cq_quantize_pack_token",
 )
+
+
+class DecodePlan(C.Structure):
+    """Mirror of `cq_decode_plan`."""
+    _fields_ = [("threads", C.c_int), ("heads_per_unit", C.c_int), ("chunks", C.c_int), ("chunk_tokens", C.c_int),
+                ("launches", C.c_int), ("lds_bytes", C.c_int), ("f16_logits", C.c_int)]
 
 
 class DecodeArgs(C.Structure):
@@ -79,6 +85,8 @@ def load() -> C.CDLL:
     lib.cq_lut_vecmat_pv.argtypes = vm
     lib.cq_decode_attn_workspace.restype = sz
     lib.cq_decode_attn_workspace.argtypes = [C.POINTER(DecodeArgs)]
+    lib.cq_decode_attn_plan.restype = C.c_int
+    lib.cq_decode_attn_plan.argtypes = [C.POINTER(DecodeArgs), C.POINTER(DecodePlan)]
     lib.cq_decode_attn.restype = i
     lib.cq_decode_attn.argtypes = [C.POINTER(DecodeArgs), vp]
     lib.cq_quantize_pack_token.restype = i

@@ -131,10 +131,12 @@ template <int BITS, int HPB, bool VTOK = false, int NT_ = 1024, bool F16K = fals
         return (cmax(cmax(KT, WTAB + cmin(VSUB, cap) * NB), cmax(RED, RED2)) + 255) / 256 * 256;
     }
     static constexpr int lds_bytes(int cap) { return region_a(cap) + FIXED + cmax(cap * SLOT, F16K ? NIBF * 4 : 0); }
+    // largest chunk whose layout fits: the whole LDS for a 1024-thread workgroup, half of it for a
+    // 512-thread workgroup (two are meant to be resident per compute unit)
     static constexpr int max_chunk() {
         int best = 64;
         for (int c = 64; c <= 16384; c += 64)
-            if (lds_bytes(c) <= kLdsMax) best = c;
+            if (lds_bytes(c) <= (kNT == 512 ? kLdsMax / 2 : kLdsMax)) best = c;
         return best;
     }
 };
@@ -535,7 +537,7 @@ __global__ __launch_bounds__(NT) void decode_kernel(DecodeGeom g) {
                         mnp[i] = __builtin_elementwise_min(mnp[i], part[5][i]);
                         mxp[i] = __builtin_elementwise_max(mxp[i], part[5][i]);
                     }
-                    *reinterpret_cast<KW*>(slot(tt)) = o;
+                    if constexpr (!MINMAX_ONLY) *reinterpret_cast<KW*>(slot(tt)) = o;
                 } else {
                 V part[6];
 #pragma unroll
@@ -1208,11 +1210,15 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
         // More units than compute units: 512-thread workgroups, two resident per compute unit, need fewer
         // instructions per unit than one 1024-thread workgroup after the other (half as many waves pay
         // the per-wave set-up, reductions and folds) - when a unit's whole layout fits half the LDS.
+        // Single launch: only if the 512-thread layout also holds all T tokens.  Chunked launch (four heads
+        // per unit): the chunks are units of their own.
         const int64_t units = static_cast<int64_t>(a->B) * a->Hkv * (G / p->hpb);
-        if (!vtok && a->force_splits == 0 && p->nsplit == 1 && units > kPairUnits && p->hpb >= 2) {
+        if (!vtok && a->force_splits == 0 && p->hpb >= 2) {
             Plan q;
             if (p->hpb == 4) plan_for<1, 4, false, 512, true>(a, &q); else plan_for<1, 2, false, 512, false>(a, &q);
-            if (q.nsplit == 1 && q.lds <= kLdsMax / 2) *p = q;
+            const bool single = p->nsplit == 1 && q.nsplit == 1 && units > kPairUnits;
+            const bool chunked = p->hpb == 4 && p->nsplit > 1 && q.nsplit > 1 && units * q.nsplit > kPairUnits;
+            if ((single || chunked) && q.lds <= kLdsMax / 2) *p = q;
         }
     } else {
         // four heads per unit need the two-pass K table; with per-token values their LDS layout
@@ -1231,8 +1237,7 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
     const int G = g.Hq / g.Hkv;
     const unsigned units = static_cast<unsigned>(g.B) * g.Hkv * (G / HPB);
     auto kmain = decode_kernel<BITS, HPB, DT, false, VTOK, NT, F16K>;
-    // the min/max pass never looks at values (the 512-thread plans are single-launch: it is never run for them)
-    auto kmm = decode_kernel<BITS, HPB, DT, true, false, 1024, false>;
+    auto kmm = decode_kernel<BITS, HPB, DT, true, false, NT, F16K>;   // the min/max pass never looks at values
     // raise the dynamic-LDS limit once per device for this instantiation
     static std::atomic<uint32_t> attr_done{0};
     int dev = 0;
@@ -1261,10 +1266,9 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
         g1.nx = g.nsplit;  // the min/max pass has no residual unit
         g1.d_nx.set(static_cast<uint32_t>(g.nsplit));
         // ... and keeps no logits, unless the table takes two passes (partial logits wait in the slots)
-        if (NT != 1024) return CQ_ERR_UNSUPPORTED;
-        g1.cap = Lay<BITS, HPB, false>::KPASS > 1 ? p.cap : 0;
-        const int lds_mm = Lay<BITS, HPB, false>::lds_bytes(g1.cap);
-        hipLaunchKernelGGL(kmm, dim3(units * g.nsplit), dim3(1024), lds_mm, st, g1);
+        g1.cap = Lay<BITS, HPB, false, NT, F16K>::KPASS > 1 ? p.cap : 0;
+        const int lds_mm = Lay<BITS, HPB, false, NT, F16K>::lds_bytes(g1.cap);
+        hipLaunchKernelGGL(kmm, dim3(units * g.nsplit), dim3(NT), lds_mm, st, g1);
         CQ_LAUNCH_CHECK();
     }
     hipLaunchKernelGGL(kmain, dim3(units * g.nx), dim3(NT), p.lds, st, gm);
@@ -1303,6 +1307,21 @@ size_t cq_decode_attn_workspace(const cq_decode_args* args) {
     cq::Plan p;
     if (cq::make_plan(args, &p) != CQ_OK) return 0;
     return p.ws_mm + p.ws_part;
+}
+
+int cq_decode_attn_plan(const cq_decode_args* args, cq_decode_plan* plan) {
+    if (!plan) return CQ_ERR_NULL;
+    cq::Plan p;
+    const int rc = cq::make_plan(args, &p);
+    if (rc != CQ_OK) return rc;
+    plan->threads = p.nt;
+    plan->heads_per_unit = p.hpb;
+    plan->chunks = p.nsplit;
+    plan->chunk_tokens = args->T > 0 ? p.chunk : 0;
+    plan->launches = p.nsplit > 1 ? 3 : 1;
+    plan->lds_bytes = p.lds;
+    plan->f16_logits = (p.nt == 512 && p.hpb == 4) ? 1 : 0;
+    return CQ_OK;
 }
 
 int cq_decode_attn(const cq_decode_args* a, cq_stream_t stream) {

@@ -225,6 +225,13 @@ class DecodeCall:
         self.args, self._ref, self._keep, self.out, self.device = a, C.byref(a), keep, out, q.device
         self.workspace_bytes = 0 if ws is None else ws.numel()
 
+    def plan(self) -> dict:
+        """What the launch will be for the prepared arguments (`cq_decode_attn_plan`): threads per
+        workgroup, query heads per workgroup, token chunks, launches, LDS bytes, packed-fp16 logits."""
+        p = _lib.DecodePlan()
+        _lib.check(self._lib.cq_decode_attn_plan(self._ref, C.byref(p)), "cq_decode_attn_plan")
+        return {name: int(getattr(p, name)) for name, _ in p._fields_}
+
     def step(self, q: torch.Tensor, k_res: torch.Tensor, v_res: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
         """Re-aim the prepared call at this decode step's query, output and (grown) residual
         window and launch.  Only pointers, R and the strides change; packed state, dtype, head

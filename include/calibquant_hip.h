@@ -184,6 +184,21 @@ typedef struct cq_decode_args {
 size_t cq_decode_attn_workspace(const cq_decode_args* args);
 int cq_decode_attn(const cq_decode_args* args, cq_stream_t stream);
 
+/* What cq_decode_attn would launch for these arguments (pointers are not
+ * looked at; host-only, no device call).  No counterpart in the reference,
+ * whose Triton kernels re-autotune per shape (calibquant.py:54-76,192-218):
+ * here the choice is a pure function of the shape, and a caller can read it. */
+typedef struct cq_decode_plan {
+    int threads;          /* threads per workgroup: 1024, or 512 with two workgroups per compute unit */
+    int heads_per_unit;   /* query heads served by one workgroup (they share a kv head) */
+    int chunks;           /* token chunks per (batch, kv head, head group); > 1: min/max launch + main launch + merge */
+    int chunk_tokens;     /* packed tokens per chunk */
+    int launches;         /* 1 or 3 */
+    int lds_bytes;        /* dynamic LDS of the main launch */
+    int f16_logits;       /* non-zero: K table entries, look-up sums and waiting logits are packed fp16 */
+} cq_decode_plan;
+int cq_decode_attn_plan(const cq_decode_args* args, cq_decode_plan* plan);
+
 /* ------------------------------------------------------------------------
  * Decode-step glue, one launch per layer and token: the (h gs d) split of
  * the fused wqkv output (patch_internvl.py:219-234), rotary embedding of the

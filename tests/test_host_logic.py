@@ -25,6 +25,40 @@ def test_library_loads_and_exports_every_declared_symbol():
     assert b"NULL" in lib.cq_strerror(-1) and lib.cq_strerror(0) == b"ok"
 
 
+def test_decode_launch_plan_is_a_function_of_the_shape():
+    """`cq_decode_attn_plan` (host only): which launch a shape gets.  Two 512-thread workgroups per compute
+    unit need a layout within half of the 160 KB LDS and more units of work than the 256 compute units;
+    packed-fp16 logits only at 1 bit with four heads per unit; chunked shapes take three launches."""
+    from calibquant_amd import _lib
+    lib = _lib.load()
+
+    def plan(B, Hq, Hkv, T, R, bits=1, v_mode=0, force_splits=0):
+        a = _lib.DecodeArgs()
+        a.dtype, a.D, a.B, a.Hq, a.Hkv, a.T, a.R, a.bits, a.v_mode, a.force_splits = 0, 128, B, Hq, Hkv, T, R, bits, v_mode, force_splits
+        p = _lib.DecodePlan()
+        assert lib.cq_decode_attn_plan(ctypes.byref(a), ctypes.byref(p)) == 0
+        return {n: getattr(p, n) for n, _ in p._fields_}
+
+    bench = plan(64, 32, 8, 3328, 128)
+    assert (bench["threads"], bench["heads_per_unit"], bench["launches"], bench["f16_logits"]) == (512, 4, 1, 1)
+    assert bench["lds_bytes"] <= 80 * 1024 and bench["chunk_tokens"] == 3328
+    small = plan(32, 32, 8, 3328, 128)                       # 256 units: one 1024-thread workgroup per compute unit
+    assert (small["threads"], small["f16_logits"], small["launches"]) == (1024, 0, 1)
+    assert plan(64, 32, 8, 3328, 128, bits=2)["threads"] == 1024
+    assert plan(64, 32, 8, 3328, 128, v_mode=1)["threads"] == 1024
+    assert plan(64, 32, 8, 3328, 128, force_splits=2) == dict(plan(64, 32, 8, 3328, 128, force_splits=2), threads=1024, launches=3)
+    two = plan(128, 16, 8, 3328, 128)                        # two heads per unit: paired, fp32 logits
+    assert (two["threads"], two["heads_per_unit"], two["f16_logits"]) == (512, 2, 0)
+    long = plan(8, 32, 8, 32768, 0)                          # chunked: the chunks are the units
+    assert long["launches"] == 3 and long["threads"] == 512 and long["chunks"] * long["chunk_tokens"] >= 32768
+    assert long["lds_bytes"] <= 80 * 1024
+    big = plan(16, 48, 8, 9984, 64)                          # six heads per kv head: three units of two heads, one launch
+    assert (big["threads"], big["heads_per_unit"], big["launches"]) == (1024, 2, 1)
+    a = _lib.DecodeArgs()
+    assert lib.cq_decode_attn_plan(ctypes.byref(a), None) < 0
+    assert lib.cq_decode_attn_plan(ctypes.byref(a), ctypes.byref(_lib.DecodePlan())) < 0   # all-zero arguments
+
+
 def test_c_abi_rejects_bad_arguments_without_touching_the_gpu():
     """Validation happens before any launch, so these calls are safe without a device."""
     from calibquant_amd import _lib
