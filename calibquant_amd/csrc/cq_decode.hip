@@ -114,9 +114,8 @@ template <int BITS, int HPB, bool VTOK = false, int NT_ = 1024, bool F16K = fals
     static constexpr int RED2 = kNW * kD * ESZ;
     // fixed small region (floats)
     static constexpr int F_WBIT = 0;                          // NB*8*HPB
-    static constexpr int F_QF = F_WBIT + NB * 8 * HPB;        // HPB*kD
-    static constexpr int F_QSZ = F_QF + HPB * kD;             // HPB*kD
-    static constexpr int F_QRAW = F_QSZ + HPB * kD;           // HPB*kD raw 16-bit q
+    static constexpr int F_QSZ = F_WBIT + NB * 8 * HPB;       // NB*HPB: zero-point sum per byte position and head
+    static constexpr int F_QRAW = F_QSZ + NB * HPB;           // HPB*kD raw 16-bit q
     static constexpr int F_RED = F_QRAW + HPB * kD / 2;       // kNW*HPB
     static constexpr int F_STAT = F_RED + kNW * RW;           // 8*HPB: per-head softmax state
     static constexpr int F_VSZ = F_STAT + 8 * HPB;            // 2*kD: value scale, zero-point (VTOK: NGRP*HPB minimum terms)
@@ -252,7 +251,6 @@ __global__ __launch_bounds__(NT) void decode_kernel(DecodeGeom g) {
     unsigned char* slots = smem + reg_a + L::FIXED;   // one slot per token of the chunk
     auto slot = [&](int t) { return slots + t * L::SLOT; };
     float* wbit = fx + L::F_WBIT;
-    float* qf = fx + L::F_QF;
     float* qsz = fx + L::F_QSZ;
     float* red = fx + L::F_RED;
 
@@ -270,6 +268,7 @@ __global__ __launch_bounds__(NT) void decode_kernel(DecodeGeom g) {
     const int hkv = static_cast<int>(vb - qn * g.d_hkv.div);
     const int b = static_cast<int>(qn);
     const int hq0 = hkv * G + hg * HPB;
+    const int nh = min(HPB, G - hg * HPB);   // query heads of this unit; the rest of its HPB heads are padding
     const int64_t bh = static_cast<int64_t>(b) * g.Hkv + hkv;
 
     const bool img_unit = split < g.nsplit && g.T > 0;
@@ -292,7 +291,7 @@ __global__ __launch_bounds__(NT) void decode_kernel(DecodeGeom g) {
     constexpr bool kVSep = (HPB * kD > kNT - kD);
     uint32_t vs_raw = 0, vz_raw = 0;
     {
-        const int h = min(tid / kD, HPB - 1), d = tid % kD;
+        const int h = min(min(tid / kD, HPB - 1), nh - 1), d = tid % kD;   // a padding head repeats the last real one
         const uint16_t* qp = static_cast<const uint16_t*>(g.q) + (static_cast<int64_t>(b) * g.Hq + hq0) * kD;
         q_raw = qp[h * kD + d];
         // the last kD threads fetch the value statistics, unless they are q threads as well
@@ -342,7 +341,6 @@ __global__ __launch_bounds__(NT) void decode_kernel(DecodeGeom g) {
         const float qraw = Cvt<DT>::to_float(q_raw);
         reinterpret_cast<uint16_t*>(fx + L::F_QRAW)[h * kD + d] = static_cast<uint16_t>(q_raw);
         const float qv = qraw * inv_sqrt_d;
-        qf[h * kD + d] = qv;
         if (n > 0) {
             const float s = Cvt<DT>::to_float(s_raw);
             const float z = Cvt<DT>::to_float(z_raw);
@@ -655,7 +653,7 @@ __global__ __launch_bounds__(NT) void decode_kernel(DecodeGeom g) {
     if constexpr (MINMAX_ONLY) {
 #pragma unroll
         for (int h = 0; h < HPB; ++h) {
-            if (n > 0 && tid == h) {
+            if (n > 0 && tid == h && h < nh) {
                 float* o = g.mm + ((static_cast<int64_t>(b) * g.Hq + hq0 + h) * g.nsplit + split) * 2;
                 o[0] = mn[h];
                 o[1] = mx[h];
@@ -709,7 +707,7 @@ __global__ __launch_bounds__(NT) void decode_kernel(DecodeGeom g) {
             if (g.nsplit > 1) {
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) {
-                    const float* p = g.mm + (static_cast<int64_t>(b) * g.Hq + hq0 + h) * g.nsplit * 2;
+                    const float* p = g.mm + (static_cast<int64_t>(b) * g.Hq + hq0 + min(h, nh - 1)) * g.nsplit * 2;
                     float a = INFINITY, z = -INFINITY;
                     for (int s = 0; s < g.nsplit; ++s) { a = fminf(a, p[2 * s]); z = fmaxf(z, p[2 * s + 1]); }
                     mn[h] = a; mx[h] = z;
@@ -1113,7 +1111,7 @@ __global__ __launch_bounds__(NT) void decode_kernel(DecodeGeom g) {
         }
         // ---- phase 7: merge / write ---------------------------------------------------------
         __syncthreads();
-        if (tid < HPB * kD) {
+        if (tid < nh * kD) {
             const int h = tid / kD, d = tid % kD;
             const float mr = stat[HPB + h], lr = stat[2 * HPB + h];
             const float mi = stat[3 * HPB + h], li = stat[4 * HPB + h];
@@ -1153,8 +1151,12 @@ __global__ void merge_kernel(const float* __restrict__ part, int nx, void* __res
     store_elem<DT>(out, row * kD + d, num / den);
 }
 
+// head groups per kv head; the last one may be partly padding (its spare heads repeat its last query head
+// and write nothing)
+static inline int ngroups(int G, int hpb) { return (G + hpb - 1) / hpb; }
+
 struct Plan {
-    int hpb, nt, nsplit, chunk, nx, cap, lds;
+    int hpb, nt, f16, nsplit, chunk, nx, cap, lds;
     size_t ws_mm, ws_part;
 };
 
@@ -1162,7 +1164,7 @@ template <int BITS, int HPB, bool VTOK, int NT = 1024, bool F16K = false>
 static void plan_for(const cq_decode_args* a, Plan* p) {
     using L = Lay<BITS, HPB, VTOK, NT, F16K>;
     const int G = a->Hq / a->Hkv;
-    const int64_t units = static_cast<int64_t>(a->B) * a->Hkv * (G / HPB);
+    const int64_t units = static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, HPB);
     const int maxc = L::max_chunk();
     int nsplit = 1;
     if (a->T > 0) {
@@ -1182,6 +1184,7 @@ static void plan_for(const cq_decode_args* a, Plan* p) {
     nsplit = a->T > 0 ? (a->T + chunk - 1) / chunk : 1;
     p->hpb = HPB;
     p->nt = NT;
+    p->f16 = F16K ? 1 : 0;
     p->nsplit = nsplit;
     p->chunk = chunk;
     p->nx = nsplit + ((nsplit > 1 && a->R > 0) ? 1 : 0);
@@ -1204,15 +1207,27 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
     if (a->v_mode != CQ_V_PER_CHANNEL && a->v_mode != CQ_V_PER_TOKEN) return CQ_ERR_UNSUPPORTED;
     const bool vtok = a->v_mode == CQ_V_PER_TOKEN;
     if (a->bits == 1) {
-        if (G % 4 == 0) vtok ? plan_for<1, 4, true>(a, p) : plan_for<1, 4, false>(a, p);
+        // G = 6, 10, ...: units of four heads with the last one half padding (two units per kv head at
+        // G = 6) do less work than units of two heads (three of them, each walking all the packed rows)
+        const bool pad4 = G % 4 == 2 && G > 4 && !vtok;
+        if (G % 4 == 0 || pad4) vtok ? plan_for<1, 4, true>(a, p) : plan_for<1, 4, false>(a, p);
         else if (G % 2 == 0) vtok ? plan_for<1, 2, true>(a, p) : plan_for<1, 2, false>(a, p);
         else vtok ? plan_for<1, 1, true>(a, p) : plan_for<1, 1, false>(a, p);
         // More units than compute units: 512-thread workgroups, two resident per compute unit, need fewer
         // instructions per unit than one 1024-thread workgroup after the other (half as many waves pay
         // the per-wave set-up, reductions and folds) - when a unit's whole layout fits half the LDS.
+        // Four heads per unit, enough units to fill the device, and T beyond the fp32 layout: the packed-fp16
+        // layout (half the bytes per waiting token) may still hold all T tokens in one launch, which saves the
+        // min/max launch's second pass over the packed K rows.
+        if (p->hpb == 4 && !vtok && a->force_splits == 0 && p->nsplit > 1 &&
+            static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, 4) >= kPairUnits * 3 / 4) {
+            Plan q;
+            plan_for<1, 4, false, 1024, true>(a, &q);
+            if (q.nsplit == 1) *p = q;
+        }
         // Single launch: only if the 512-thread layout also holds all T tokens.  Chunked launch (four heads
         // per unit): the chunks are units of their own.
-        const int64_t units = static_cast<int64_t>(a->B) * a->Hkv * (G / p->hpb);
+        const int64_t units = static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, p->hpb);
         if (!vtok && a->force_splits == 0 && p->hpb >= 2) {
             Plan q;
             if (p->hpb == 4) plan_for<1, 4, false, 512, true>(a, &q); else plan_for<1, 2, false, 512, false>(a, &q);
@@ -1223,11 +1238,11 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
     } else {
         // four heads per unit need the two-pass K table; with per-token values their LDS layout
         // would not hold a 3 328-token chunk, so that mode keeps two heads per unit
-        if (G % 4 == 0 && !vtok) plan_for<2, 4, false>(a, p);
+        if ((G % 4 == 0 || (G % 4 == 2 && G > 4)) && !vtok) plan_for<2, 4, false>(a, p);
         else if (G % 2 == 0) vtok ? plan_for<2, 2, true>(a, p) : plan_for<2, 2, false>(a, p);
         else vtok ? plan_for<2, 1, true>(a, p) : plan_for<2, 1, false>(a, p);
     }
-    const int64_t blocks = static_cast<int64_t>(a->B) * a->Hkv * (G / p->hpb) * p->nx;
+    const int64_t blocks = static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, p->hpb) * p->nx;
     if (blocks > 0x7fffffff) return CQ_ERR_SHAPE;
     return CQ_OK;
 }
@@ -1235,7 +1250,7 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
 template <int BITS, int HPB, typename DT, bool VTOK, int NT = 1024, bool F16K = false>
 static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
     const int G = g.Hq / g.Hkv;
-    const unsigned units = static_cast<unsigned>(g.B) * g.Hkv * (G / HPB);
+    const unsigned units = static_cast<unsigned>(g.B) * g.Hkv * ngroups(G, HPB);
     auto kmain = decode_kernel<BITS, HPB, DT, false, VTOK, NT, F16K>;
     auto kmm = decode_kernel<BITS, HPB, DT, true, false, NT, F16K>;   // the min/max pass never looks at values
     // raise the dynamic-LDS limit once per device for this instantiation
@@ -1258,7 +1273,7 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
     }
     DecodeGeom gm = g;
     gm.G = G;
-    gm.d_ng.set(static_cast<uint32_t>(G / HPB));
+    gm.d_ng.set(static_cast<uint32_t>(ngroups(G, HPB)));
     gm.d_nx.set(static_cast<uint32_t>(g.nx));
     gm.d_hkv.set(static_cast<uint32_t>(g.Hkv));
     if (g.nsplit > 1) {
@@ -1286,6 +1301,7 @@ static int dispatch(const DecodeGeom& g, const Plan& p, int bits, hipStream_t st
     if (bits == 1) {
         if constexpr (!VTOK) {
             if (p.hpb == 4 && p.nt == 512) return launch<1, 4, DT, false, 512, true>(g, p, st);
+            if (p.hpb == 4 && p.f16) return launch<1, 4, DT, false, 1024, true>(g, p, st);
             if (p.hpb == 2 && p.nt == 512) return launch<1, 2, DT, false, 512, false>(g, p, st);
         }
         if (p.hpb == 4) return launch<1, 4, DT, VTOK>(g, p, st);
@@ -1320,7 +1336,7 @@ int cq_decode_attn_plan(const cq_decode_args* args, cq_decode_plan* plan) {
     plan->chunk_tokens = args->T > 0 ? p.chunk : 0;
     plan->launches = p.nsplit > 1 ? 3 : 1;
     plan->lds_bytes = p.lds;
-    plan->f16_logits = (p.nt == 512 && p.hpb == 4) ? 1 : 0;
+    plan->f16_logits = p.f16;
     return CQ_OK;
 }
 

@@ -221,6 +221,8 @@ PAIRED = [
     (20, 16, 8, 1500, 130, 3, "bf16", True, True),      # two heads per unit: fp32 logits
     (17, 48, 8, 1000, 33, 0, "fp16", False, True),      # six q heads per kv head: three units of two heads
     (20, 32, 8, 0, 200, 0, "bf16", False, True),        # window only
+    (12, 32, 8, 5000, 64, 0, "bf16", False, True),      # 192 units, T beyond the fp32 layout: one launch, packed-fp16 logits
+    (8, 48, 8, 5000, 64, 3, "fp16", False, True),       # six q heads per kv head: two units of four heads, the second half padding
     (4, 32, 8, 9000, 100, 7, "bf16", False, True),      # chunked: 64 units x 8 chunks, min/max launch + merge
     (4, 32, 8, 9000, 0, 0, "fp16", True, True),
 ]

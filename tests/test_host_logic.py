@@ -52,8 +52,10 @@ def test_decode_launch_plan_is_a_function_of_the_shape():
     long = plan(8, 32, 8, 32768, 0)                          # chunked: the chunks are the units
     assert long["launches"] == 3 and long["threads"] == 512 and long["chunks"] * long["chunk_tokens"] >= 32768
     assert long["lds_bytes"] <= 80 * 1024
-    big = plan(16, 48, 8, 9984, 64)                          # six heads per kv head: three units of two heads, one launch
-    assert (big["threads"], big["heads_per_unit"], big["launches"]) == (1024, 2, 1)
+    big = plan(16, 48, 8, 9984, 64)     # six heads per kv head: two units of four (the second half padding); one launch
+    assert (big["threads"], big["heads_per_unit"], big["launches"], big["f16_logits"]) == (1024, 4, 1, 1)   # needs packed-fp16 logits
+    assert big["lds_bytes"] <= 160 * 1024
+    assert plan(16, 48, 8, 9984, 64, v_mode=1)["heads_per_unit"] == 2
     a = _lib.DecodeArgs()
     assert lib.cq_decode_attn_plan(ctypes.byref(a), None) < 0
     assert lib.cq_decode_attn_plan(ctypes.byref(a), ctypes.byref(_lib.DecodePlan())) < 0   # all-zero arguments
