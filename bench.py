@@ -399,8 +399,7 @@ def main():
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
-        # fp32 accumulation throughout; the paired 512-thread launch sums its K look-ups in packed fp16
-        "dtype": "f32+f16" if plan["f16_logits"] else "f32",
+        "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": a.workload, "batch": B, "q_heads": Hq, "kv_heads": Hkv, "head_dim": D,
                    "kv_packed_tokens": T, "kv_residual_rows": R, "bits": a.bits, "storage_dtype": "bf16",

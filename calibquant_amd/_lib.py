@@ -23,7 +23,7 @@ SYMBOLS = (
 class DecodePlan(C.Structure):
     """Mirror of `cq_decode_plan`."""
     _fields_ = [("threads", C.c_int), ("heads_per_unit", C.c_int), ("chunks", C.c_int), ("chunk_tokens", C.c_int),
-                ("launches", C.c_int), ("lds_bytes", C.c_int), ("f16_logits", C.c_int)]
+                ("launches", C.c_int), ("lds_bytes", C.c_int), ("register_logits", C.c_int)]
 
 
 class DecodeArgs(C.Structure):

@@ -43,6 +43,8 @@ constexpr int kD = 128;
 constexpr int kPF = 4;             // 16-byte loads kept in flight per thread and stream
 constexpr int kLdsMax = 160 * 1024;
 constexpr int kPairUnits = 256;    // compute units of the device this is laid out for
+constexpr int kRegPair = 8;        // rounds of logits a thread of a 512-thread workgroup keeps in registers (4 096 tokens)
+constexpr int kRegLong = 10;       // ... of a 1024-thread workgroup that holds a long chunk in one launch (10 240 tokens)
 constexpr float kLog2e = 1.4426950408889634f;
 
 template <int N> struct alignas(N * 4) Vec { float v[N]; };
@@ -79,10 +81,12 @@ constexpr int cmin(int a, int b) { return a < b ? a : b; }
 // codes in little-endian 32-bit words, first channel in the lowest bits) instead of per
 // channel.  A token slot then also carries the token's group scales, and every channel
 // group has its own subset-sum tables.
-// F16K: the K table entries, the look-up sums and the logits waiting in the token slots are packed
-// fp16 (half the LDS bytes, so that two 512-thread workgroups fit a compute unit's LDS); the
-// reference's own look-up kernel stores its logits as fp16 as well (calibquant.py:104-111).
-template <int BITS, int HPB, bool VTOK = false, int NT_ = 1024, bool F16K = false> struct Lay {
+// REGL > 0: a thread keeps the logits of its tokens (at most REGL rounds of kNT tokens) in registers
+// until the block's min / max are known and writes only e = exp(.) to the token slots, as packed fp16:
+// the slots take half the bytes, which is what lets two 512-thread workgroups share a compute unit's
+// LDS (with the K table built for half of the byte positions at a time), or one 1024-thread workgroup
+// hold a chunk of 9 984 tokens.
+template <int BITS, int HPB, bool VTOK = false, int NT_ = 1024, int REGL = 0> struct Lay {
     static constexpr int kNT = NT_;                 // threads per workgroup
     static constexpr int kNW = kNT / kWave;         // waves per workgroup
     static constexpr int kResTile = kNT / 8;        // residual rows per tile (8 lanes per row)
@@ -94,17 +98,19 @@ template <int BITS, int HPB, bool VTOK = false, int NT_ = 1024, bool F16K = fals
     static constexpr int ESZ = HPB * 4;             // bytes per fp32 table entry / logits slot
     static constexpr int HW = HPB >= 2 ? HPB / 2 : 1;   // 32-bit words per packed-fp16 entry
     static constexpr int ESZH = HW * 4;             // bytes per packed-fp16 table entry
-    // The byte-indexed K table covers NBP byte positions at a time: all of them when that fits
-    // 64 KB, else half of them in each of two passes over the chunk's rows (one 16-byte piece
-    // of a 2-bit row per pass), the first pass's partial logits waiting in the token slots.
-    static constexpr int KESZ = F16K ? ESZH : ESZ;  // bytes per K table entry and per waiting logits slot
-    static constexpr int KPASS = (NB * 256 * KESZ > 64 * 1024) ? 2 : 1;
+    // The byte-indexed K table covers NBP byte positions at a time: all of them when that fits the
+    // table's share of the LDS (64 KB; 32 KB for a 512-thread workgroup), else half of them in each of
+    // two passes over the chunk's rows, the first pass's partial logits waiting in the token slots or,
+    // with REGL, in registers.
+    static constexpr int KTMAX = (NT_ == 512 ? 32 : 64) * 1024;
+    static constexpr int KPASS = (NB * 256 * ESZ > KTMAX) ? 2 : 1;
     static constexpr int NBP = NB / KPASS;          // byte positions per pass
-    static constexpr int PPP = BITS / KPASS;        // 16-byte pieces of a row per pass
-    static constexpr int KT = NBP * 256 * KESZ;     // K table bytes
-    static_assert(!F16K || (KPASS == 1 && !VTOK && HPB >= 2), "packed-fp16 logits: one table pass, per-channel values");
-    static_assert(KPASS == 1 || (KPASS == 2 && BITS == 2), "a pass consumes whole 16-byte pieces");
-    static constexpr int SLOT = VTOK ? 16 : KESZ;   // bytes per token slot: logits, later e (+ 4 group scales)
+    static constexpr int WPP = NBP / 4;             // 32-bit words of a row per pass
+    static constexpr int PCS = (WPP + 3) / 4;       // 16-byte pieces of a row a pass looks at
+    static constexpr int KT = NBP * 256 * ESZ;      // K table bytes
+    static_assert(NB * 256 * ESZ <= 2 * KTMAX, "at most two table passes");
+    static_assert(!(REGL > 0 && VTOK), "logits in registers: per-channel values only");
+    static constexpr int SLOT = VTOK ? 16 : (REGL > 0 ? ESZH : ESZ);   // bytes per token slot: logits, later e (+ 4 group scales)
     static constexpr int NGRP = VTOK ? kD / 32 : 1; // channel groups with tables of their own
     static constexpr int WTAB = kNW * NGRP * GPW * 16 * ESZH;
     static constexpr int RW = cmax(3 * HPB, VTOK ? (NGRP + 1) * HPB : 0);   // per-wave partials: min/max + masked max, or the closing sums
@@ -120,22 +126,22 @@ template <int BITS, int HPB, bool VTOK = false, int NT_ = 1024, bool F16K = fals
     static constexpr int F_STAT = F_RED + kNW * RW;           // 8*HPB: per-head softmax state
     static constexpr int F_VSZ = F_STAT + 8 * HPB;            // 2*kD: value scale, zero-point (VTOK: NGRP*HPB minimum terms)
     static constexpr int F_NIB = F_VSZ + 2 * kD;              // NB*32*HPB: nibble tables
-    // (F16K: the nibble tables live in the token slots, which are first written after the table build)
+    // (REGL: the nibble tables live in the token slots, which are first written after the last table pass)
     static constexpr int NIBF = NB * 32 * HPB;
-    static constexpr int F_SRES = F_NIB + (F16K ? 0 : NIBF);  // kResTile*HPB
+    static constexpr int F_SRES = F_NIB + (REGL > 0 ? 0 : NIBF);  // kResTile*HPB
     static constexpr int F_PRES = F_SRES + kResTile * HPB;    // kResTile*HPB
     static constexpr int F_END = F_PRES + kResTile * HPB;
     static constexpr int FIXED = ((F_END * 4 + 255) / 256) * 256;
     static constexpr int region_a(int cap) {
         return (cmax(cmax(KT, WTAB + cmin(VSUB, cap) * NB), cmax(RED, RED2)) + 255) / 256 * 256;
     }
-    static constexpr int lds_bytes(int cap) { return region_a(cap) + FIXED + cmax(cap * SLOT, F16K ? NIBF * 4 : 0); }
+    static constexpr int lds_bytes(int cap) { return region_a(cap) + FIXED + cmax(cap * SLOT, REGL > 0 ? NIBF * 4 : 0); }
     // largest chunk whose layout fits: the whole LDS for a 1024-thread workgroup, half of it for a
     // 512-thread workgroup (two are meant to be resident per compute unit)
     static constexpr int max_chunk() {
         int best = 64;
         for (int c = 64; c <= 16384; c += 64)
-            if (lds_bytes(c) <= (kNT == 512 ? kLdsMax / 2 : kLdsMax)) best = c;
+            if (lds_bytes(c) <= (kNT == 512 ? kLdsMax / 2 : kLdsMax) && (REGL == 0 || c <= REGL * kNT)) best = c;
         return best;
     }
 };
@@ -238,9 +244,9 @@ __device__ __forceinline__ uint32_t pack_f16(float a, float b) {
     return __builtin_bit_cast(uint32_t, h);
 }
 
-template <int BITS, int HPB, typename DT, bool MINMAX_ONLY, bool VTOK = false, int NT = 1024, bool F16K = false>
+template <int BITS, int HPB, typename DT, bool MINMAX_ONLY, bool VTOK = false, int NT = 1024, int REGL = 0>
 __global__ __launch_bounds__(NT) void decode_kernel(DecodeGeom g) {
-    using L = Lay<BITS, HPB, VTOK, NT, F16K>;
+    using L = Lay<BITS, HPB, VTOK, NT, REGL>;
     using V = Vec<HPB>;
     constexpr int NB = L::NB;
     constexpr int kNT = L::kNT, kNW = L::kNW, kResTile = L::kResTile;
@@ -385,37 +391,28 @@ __global__ __launch_bounds__(NT) void decode_kernel(DecodeGeom g) {
     float mn[HPB], mx[HPB];
 #pragma unroll
     for (int h = 0; h < HPB; ++h) { mn[h] = INFINITY; mx[h] = -INFINITY; }
-    // F16K: running min / max of the packed logits, two heads per register
-    f16x2_t mnp[L::HW], mxp[L::HW];
+    // REGL: the logits of this thread's tokens, round r = token tid + r * kNT
+    V lg[REGL > 0 ? REGL : 1];
+    // logits (later: calibrated, masked logits) of a token: in its slot, or in the thread's registers
+    auto load_logits = [&](int rd, int tt) {
+        if constexpr (REGL > 0) return lg[rd];
+        else return *reinterpret_cast<const V*>(slot(tt));
+    };
+    auto store_logits = [&](int rd, int tt, const V& w) {
+        if constexpr (REGL > 0) lg[rd] = w;
+        else *reinterpret_cast<V*>(slot(tt)) = w;
+    };
+    // f(round, token) for the thread's tokens below lim; with REGL the rounds are unrolled so that
+    // lg[] is indexed by constants
+    auto for_my_tokens = [&](int lim, auto&& f) {
+        if constexpr (REGL > 0) {
 #pragma unroll
-    for (int k = 0; k < L::HW; ++k) {
-        mnp[k] = f16x2_t{static_cast<_Float16>(INFINITY), static_cast<_Float16>(INFINITY)};
-        mxp[k] = f16x2_t{static_cast<_Float16>(-INFINITY), static_cast<_Float16>(-INFINITY)};
-    }
-    using KW = Words<L::HW>;   // a packed-fp16 entry: the unit's heads, two per word
-    // logits (later: calibrated, masked logits) waiting in a token's slot
-    auto load_logits = [&](int tt) {
-        V w;
-        if constexpr (F16K) {
-            const KW r = *reinterpret_cast<const KW*>(slot(tt));
-#pragma unroll
-            for (int h = 0; h < HPB; ++h) {
-                const f16x2_t pr = __builtin_bit_cast(f16x2_t, r.w[h >> 1]);
-                w.v[h] = static_cast<float>((h & 1) ? pr.y : pr.x);
+            for (int rd = 0; rd < REGL; ++rd) {
+                const int tt = tid + rd * kNT;
+                if (tt < lim) f(rd, tt);
             }
         } else {
-            w = *reinterpret_cast<const V*>(slot(tt));
-        }
-        return w;
-    };
-    auto store_logits = [&](int tt, const V& w) {
-        if constexpr (F16K) {
-            KW r;
-#pragma unroll
-            for (int k = 0; k < L::HW; ++k) r.w[k] = pack_f16(w.v[2 * k], w.v[2 * k + 1]);
-            *reinterpret_cast<KW*>(slot(tt)) = r;
-        } else {
-            *reinterpret_cast<V*>(slot(tt)) = w;
+            for (int tt = tid; tt < lim; tt += kNT) f(0, tt);
         }
     };
     // First block of packed V rows: half of it is requested here, behind the packed K rows, the
@@ -432,7 +429,7 @@ __global__ __launch_bounds__(NT) void decode_kernel(DecodeGeom g) {
         // ---- phase 2: byte table = high-nibble table + low-nibble table ----------------
         // nibble tables: entry (j, half, v) = sum of the per-bit weights v selects; the
         // zero-point sum of the byte position is folded into the high half.
-        V* nib = F16K ? reinterpret_cast<V*>(slots) : reinterpret_cast<V*>(fx + L::F_NIB);   // [half*16 + value][byte position]
+        V* nib = REGL > 0 ? reinterpret_cast<V*>(slots) : reinterpret_cast<V*>(fx + L::F_NIB);   // [half*16 + value][byte position]
         V* ktab = reinterpret_cast<V*>(regA);           // [byte value][byte position]
         for (int e = tid; e < NB * 32; e += kNT) {
             const int j = e % NB, half = (e / NB) >> 4, v = (e / NB) & 15;
@@ -468,25 +465,27 @@ __global__ __launch_bounds__(NT) void decode_kernel(DecodeGeom g) {
         const uint32_t bsel = (0x03020100u ^ (0x01010101u * (skew & 3)));
         uint32_t pofs[NBP];   // byte offset of position k ^ skew inside a table row
 #pragma unroll
-        for (int k = 0; k < NBP; ++k) pofs[k] = (k ^ skew) * L::KESZ;
+        for (int k = 0; k < NBP; ++k) pofs[k] = (k ^ skew) * L::ESZ;
         const unsigned char* ktab_b = regA;
         // With 256-byte table rows the address of a look-up is two bytes side by side, the
         // byte value above the position offset: one byte permute builds it from the row word
         // and a word holding four position offsets.
-        constexpr bool kPermAddr = (NBP * L::KESZ == 256) && !F16K;
+        constexpr bool kPermAddr = (NBP * L::ESZ == 256);
         uint32_t pofs4[NBP / 4];
 #pragma unroll
         for (int i = 0; i < NBP / 4; ++i)
             pofs4[i] = pofs[4 * i] | (pofs[4 * i + 1] << 8) | (pofs[4 * i + 2] << 16) | (pofs[4 * i + 3] << 24);
-        // c: the L::PPP pieces of the row that pass P covers
-        auto token_logits = [&](auto pass_c, int tt, const uint4* c) {
+        // c: the L::PCS 16-byte pieces of the row that pass P looks at; rd: the token's round (REGL)
+        auto token_logits = [&](auto pass_c, int rd, int tt, const uint4* c) {
             constexpr int P = decltype(pass_c)::value;
             if (tt < n) {
+                constexpr int WO = (P * L::WPP) % 4;   // the pass's first word inside its first piece
                 uint32_t w[NW32];
 #pragma unroll
-                for (int i = 0; i < L::PPP; ++i) {
-                    w[4 * i + 0] = c[i].x; w[4 * i + 1] = c[i].y;
-                    w[4 * i + 2] = c[i].z; w[4 * i + 3] = c[i].w;
+                for (int i = 0; i < NW32; ++i) {
+                    const uint4& pc = c[(WO + i) / 4];
+                    const int k4 = (WO + i) % 4;
+                    w[i] = k4 == 0 ? pc.x : k4 == 1 ? pc.y : k4 == 2 ? pc.z : pc.w;
                 }
 #pragma unroll
                 for (int st = 0; (1 << st) < NW32; ++st) {   // word i <- word i ^ (skew / 4)
@@ -501,42 +500,6 @@ __global__ __launch_bounds__(NT) void decode_kernel(DecodeGeom g) {
 #pragma unroll
                 for (int i = 0; i < NW32; ++i) wds[i] = __builtin_amdgcn_perm(w[i], w[i], bsel);
                 // balanced-tree sum with a small stack of partial sums (level l holds 2^l terms)
-                if constexpr (F16K) {
-                    f16x2_t part[6][L::HW];
-#pragma unroll
-                    for (int k = 0; k < NBP; ++k) {
-                        // absolute LDS address (the table starts at 0): table row of the byte value, position inside
-                        const uint32_t byte = (wds[k >> 2] >> (8 * (k & 3))) & 0xffu;
-                        const KW r = lds_words<L::HW>(byte * (NBP * L::KESZ) + pofs[k]);
-                        f16x2_t cur[L::HW];
-#pragma unroll
-                        for (int i = 0; i < L::HW; ++i) cur[i] = __builtin_bit_cast(f16x2_t, r.w[i]);
-#pragma unroll
-                        for (int l = 0; l < 6; ++l) {
-                            if ((k >> l) & 1) {
-#pragma unroll
-                                for (int i = 0; i < L::HW; ++i) cur[i] += part[l][i];
-                            } else {
-#pragma unroll
-                                for (int i = 0; i < L::HW; ++i) part[l][i] = cur[i];
-                                break;
-                            }
-                        }
-                        if (k == NBP - 1) {
-#pragma unroll
-                            for (int i = 0; i < L::HW; ++i) part[5][i] = cur[i];
-                        }
-                        if ((k & 7) == 7) __builtin_amdgcn_sched_barrier(0);
-                    }
-                    KW o;
-#pragma unroll
-                    for (int i = 0; i < L::HW; ++i) {
-                        o.w[i] = __builtin_bit_cast(uint32_t, part[5][i]);
-                        mnp[i] = __builtin_elementwise_min(mnp[i], part[5][i]);
-                        mxp[i] = __builtin_elementwise_max(mxp[i], part[5][i]);
-                    }
-                    if constexpr (!MINMAX_ONLY) *reinterpret_cast<KW*>(slot(tt)) = o;
-                } else {
                 V part[6];
 #pragma unroll
                 for (int k = 0; k < NBP; ++k) {
@@ -567,20 +530,20 @@ __global__ __launch_bounds__(NT) void decode_kernel(DecodeGeom g) {
                 }
                 V acc = part[5];
                 if constexpr (P > 0) {   // add the earlier pass's partial
-                    const V prev = *reinterpret_cast<const V*>(slot(tt));
+                    const V prev = load_logits(rd, tt);
 #pragma unroll
                     for (int h = 0; h < HPB; ++h) acc.v[h] += prev.v[h];
                 }
-                if constexpr (!MINMAX_ONLY || P + 1 < L::KPASS) *reinterpret_cast<V*>(slot(tt)) = acc;
+                if constexpr (!MINMAX_ONLY || P + 1 < L::KPASS) store_logits(rd, tt, acc);
                 if constexpr (P + 1 == L::KPASS) {
 #pragma unroll
                     for (int h = 0; h < HPB; ++h) { mn[h] = fminf(mn[h], acc.v[h]); mx[h] = fmaxf(mx[h], acc.v[h]); }
-                }
                 }
             }
         };
         auto k_pass = [&](auto pass_c) {
             constexpr int P = decltype(pass_c)::value;
+            constexpr int kP0 = (P * L::WPP) / 4;   // first 16-byte piece of a row the pass looks at
             // byte table of the pass's positions = high-nibble table + low-nibble table
             for (int e = tid; e < NBP * 256; e += kNT) {
                 const int j = P * NBP + e % NBP, v = e / NBP;
@@ -589,14 +552,7 @@ __global__ __launch_bounds__(NT) void decode_kernel(DecodeGeom g) {
                 V o;
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) o.v[h] = hi.v[h] + lo.v[h];
-                if constexpr (F16K) {
-                    KW o16;
-#pragma unroll
-                    for (int i = 0; i < L::HW; ++i) o16.w[i] = pack_f16(o.v[2 * i], o.v[2 * i + 1]);
-                    reinterpret_cast<KW*>(regA)[e] = o16;
-                } else {
-                    ktab[e] = o;
-                }
+                ktab[e] = o;
             }
             __syncthreads();
             // first batch: rows already in registers; each consumed round of the last pass frees
@@ -604,7 +560,7 @@ __global__ __launch_bounds__(NT) void decode_kernel(DecodeGeom g) {
             // (written out round by round with constant indices so vc stays in registers)
 #define CQ_K_ROUND(R)                                                                         \
             if constexpr (L::KR > (R)) {                                                      \
-                token_logits(pass_c, tid + (R) * kNT, kc[(R)] + P * L::PPP);                  \
+                token_logits(pass_c, (R), tid + (R) * kNT, kc[(R)] + kP0);                    \
                 if constexpr (!MINMAX_ONLY && P + 1 == L::KPASS) {                            \
                     if constexpr (kVEarly + (R) * BITS < kPF) request_v(kVEarly + (R) * BITS);    \
                     if constexpr (BITS == 2 && kVEarly + (R) * BITS + 1 < kPF) request_v(kVEarly + (R) * BITS + 1); \
@@ -616,29 +572,41 @@ __global__ __launch_bounds__(NT) void decode_kernel(DecodeGeom g) {
             CQ_K_ROUND(3)
 #undef CQ_K_ROUND
             static_assert(L::KR <= 4, "rounds are written out up to 4");
-            uint4 kx[L::KR][L::PPP];   // rows beyond the first batch: this pass's pieces only
-            for (int tb = kNT * L::KR; tb < n; tb += kNT * L::KR) {
+            uint4 kx[L::KR][L::PCS];   // rows beyond the first batch: this pass's pieces only
+            if constexpr (REGL > 0) {
+                // batches written out, so that the logits' registers are indexed by constants
 #pragma unroll
-                for (int r = 0; r < L::KR; ++r) {
-                    const int tt = min(tb + tid + r * kNT, n - 1);
+                for (int ob = 1; ob < (REGL + L::KR - 1) / L::KR; ++ob) {
+                    const int tb = ob * kNT * L::KR;
+                    if (tb < n) {
 #pragma unroll
-                    for (int i = 0; i < L::PPP; ++i) kx[r][i] = ckp[static_cast<int64_t>(tt) * BITS + P * L::PPP + i];
+                        for (int r = 0; r < L::KR; ++r) {
+                            const int tt = min(tb + tid + r * kNT, n - 1);
+#pragma unroll
+                            for (int i = 0; i < L::PCS; ++i) kx[r][i] = ckp[static_cast<int64_t>(tt) * BITS + kP0 + i];
+                        }
+#pragma unroll
+                        for (int r = 0; r < L::KR; ++r)
+                            if (ob * L::KR + r < REGL) token_logits(pass_c, ob * L::KR + r, tb + tid + r * kNT, kx[r]);
+                    }
                 }
+            } else {
+                for (int tb = kNT * L::KR; tb < n; tb += kNT * L::KR) {
 #pragma unroll
-                for (int r = 0; r < L::KR; ++r) token_logits(pass_c, tb + tid + r * kNT, kx[r]);
+                    for (int r = 0; r < L::KR; ++r) {
+                        const int tt = min(tb + tid + r * kNT, n - 1);
+#pragma unroll
+                        for (int i = 0; i < L::PCS; ++i) kx[r][i] = ckp[static_cast<int64_t>(tt) * BITS + kP0 + i];
+                    }
+#pragma unroll
+                    for (int r = 0; r < L::KR; ++r) token_logits(pass_c, 0, tb + tid + r * kNT, kx[r]);
+                }
             }
         };
         k_pass(std::integral_constant<int, 0>{});
         if constexpr (L::KPASS == 2) {
             __syncthreads();   // every wave is done with the first pass's table
             k_pass(std::integral_constant<int, 1>{});
-        }
-    }
-    if constexpr (F16K) {
-#pragma unroll
-        for (int h = 0; h < HPB; ++h) {
-            mn[h] = static_cast<float>((h & 1) ? mnp[h >> 1].y : mnp[h >> 1].x);
-            mx[h] = static_cast<float>((h & 1) ? mxp[h >> 1].y : mxp[h >> 1].x);
         }
     }
     if (n > 0) {   // one reduction for both: max of (-min, max)
@@ -730,17 +698,16 @@ __global__ __launch_bounds__(NT) void decode_kernel(DecodeGeom g) {
                 float lm[HPB];
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) lm[h] = -INFINITY;
-                for (int tt = tid; tt < n; tt += kNT) {
-                    V w = load_logits(tt);
+                for_my_tokens(n, [&](int rd, int tt) {
+                    V w = load_logits(rd, tt);
                     const float mv = mk[tt];
 #pragma unroll
                     for (int h = 0; h < HPB; ++h) {
                         w.v[h] = (w.v[h] - mn[h]) * slope[h] + tmin[h] + mv;
-                        if constexpr (F16K) w.v[h] = static_cast<float>(static_cast<_Float16>(w.v[h]));   // as it will wait in the slot
                         lm[h] = fmaxf(lm[h], w.v[h]);
                     }
-                    store_logits(tt, w);
-                }
+                    store_logits(rd, tt, w);
+                });
                 block_max<HPB, kNW>(lm, red + kNW * 2 * HPB);   // the first reduction's words may still be read
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) { m_img[h] = lm[h]; slope[h] = 1.0f; tmin[h] = 0.f; mn[h] = 0.f; }
@@ -766,11 +733,11 @@ __global__ __launch_bounds__(NT) void decode_kernel(DecodeGeom g) {
             float cma[VTOK ? L::NGRP * HPB : 1];   // sum_t e[t][h] * minimum[t][group], kept [group][head]
 #pragma unroll
             for (int i = 0; i < (VTOK ? L::NGRP * HPB : 1); ++i) cma[i] = 0.f;
-            for (int tt = tid; tt < npad; tt += kNT) {
+            for_my_tokens(npad, [&](int rd, int tt) {
                 float e[4] = {0.f, 0.f, 0.f, 0.f};
                 uint32_t sc2[2] = {0u, 0u};   // the token's group scales as fp16
                 if (tt < n) {
-                    const V w = load_logits(tt);
+                    const V w = load_logits(rd, tt);
 #pragma unroll
                     for (int h = 0; h < HPB; ++h) {
                         // (w - mn) first: with a degenerate logit range the slope is ~1e8 and only the exact
@@ -796,7 +763,7 @@ __global__ __launch_bounds__(NT) void decode_kernel(DecodeGeom g) {
                 if constexpr (L::HW == 2) hw.w[1] = pack_f16(e[2], e[3]);
                 *reinterpret_cast<HWv*>(slot(tt)) = hw;
                 if constexpr (VTOK) *reinterpret_cast<uint2*>(slot(tt) + 8) = make_uint2(sc2[0], sc2[1]);
-            }
+            });
             // The sums of e (and of e * minimum) are only needed at the very end: each thread
             // keeps its partial through the packed-V phase and the fold rides on that phase's
             // closing barriers.
@@ -1156,13 +1123,13 @@ __global__ void merge_kernel(const float* __restrict__ part, int nx, void* __res
 static inline int ngroups(int G, int hpb) { return (G + hpb - 1) / hpb; }
 
 struct Plan {
-    int hpb, nt, f16, nsplit, chunk, nx, cap, lds;
+    int hpb, nt, regl, nsplit, chunk, nx, cap, lds;
     size_t ws_mm, ws_part;
 };
 
-template <int BITS, int HPB, bool VTOK, int NT = 1024, bool F16K = false>
+template <int BITS, int HPB, bool VTOK, int NT = 1024, int REGL = 0>
 static void plan_for(const cq_decode_args* a, Plan* p) {
-    using L = Lay<BITS, HPB, VTOK, NT, F16K>;
+    using L = Lay<BITS, HPB, VTOK, NT, REGL>;
     const int G = a->Hq / a->Hkv;
     const int64_t units = static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, HPB);
     const int maxc = L::max_chunk();
@@ -1184,7 +1151,7 @@ static void plan_for(const cq_decode_args* a, Plan* p) {
     nsplit = a->T > 0 ? (a->T + chunk - 1) / chunk : 1;
     p->hpb = HPB;
     p->nt = NT;
-    p->f16 = F16K ? 1 : 0;
+    p->regl = REGL;
     p->nsplit = nsplit;
     p->chunk = chunk;
     p->nx = nsplit + ((nsplit > 1 && a->R > 0) ? 1 : 0);
@@ -1216,13 +1183,13 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
         // More units than compute units: 512-thread workgroups, two resident per compute unit, need fewer
         // instructions per unit than one 1024-thread workgroup after the other (half as many waves pay
         // the per-wave set-up, reductions and folds) - when a unit's whole layout fits half the LDS.
-        // Four heads per unit, enough units to fill the device, and T beyond the fp32 layout: the packed-fp16
-        // layout (half the bytes per waiting token) may still hold all T tokens in one launch, which saves the
-        // min/max launch's second pass over the packed K rows.
+        // Four heads per unit, enough units to fill the device, and T beyond the layout with fp32 logits in
+        // the token slots: with the logits in registers (half the bytes per token slot) the layout may still
+        // hold all T tokens in one launch, which saves the min/max launch's second pass over the packed K rows.
         if (p->hpb == 4 && !vtok && a->force_splits == 0 && p->nsplit > 1 &&
             static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, 4) >= kPairUnits * 3 / 4) {
             Plan q;
-            plan_for<1, 4, false, 1024, true>(a, &q);
+            plan_for<1, 4, false, 1024, kRegLong>(a, &q);
             if (q.nsplit == 1) *p = q;
         }
         // Single launch: only if the 512-thread layout also holds all T tokens.  Chunked launch (four heads
@@ -1230,7 +1197,7 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
         const int64_t units = static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, p->hpb);
         if (!vtok && a->force_splits == 0 && p->hpb >= 2) {
             Plan q;
-            if (p->hpb == 4) plan_for<1, 4, false, 512, true>(a, &q); else plan_for<1, 2, false, 512, false>(a, &q);
+            if (p->hpb == 4) plan_for<1, 4, false, 512, kRegPair>(a, &q); else plan_for<1, 2, false, 512, 0>(a, &q);
             const bool single = p->nsplit == 1 && q.nsplit == 1 && units > kPairUnits;
             const bool chunked = p->hpb == 4 && p->nsplit > 1 && q.nsplit > 1 && units * q.nsplit > kPairUnits;
             if ((single || chunked) && q.lds <= kLdsMax / 2) *p = q;
@@ -1247,12 +1214,12 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
     return CQ_OK;
 }
 
-template <int BITS, int HPB, typename DT, bool VTOK, int NT = 1024, bool F16K = false>
+template <int BITS, int HPB, typename DT, bool VTOK, int NT = 1024, int REGL = 0>
 static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
     const int G = g.Hq / g.Hkv;
     const unsigned units = static_cast<unsigned>(g.B) * g.Hkv * ngroups(G, HPB);
-    auto kmain = decode_kernel<BITS, HPB, DT, false, VTOK, NT, F16K>;
-    auto kmm = decode_kernel<BITS, HPB, DT, true, false, NT, F16K>;   // the min/max pass never looks at values
+    auto kmain = decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL>;
+    auto kmm = decode_kernel<BITS, HPB, DT, true, false, NT, REGL>;   // the min/max pass never looks at values
     // raise the dynamic-LDS limit once per device for this instantiation
     static std::atomic<uint32_t> attr_done{0};
     int dev = 0;
@@ -1281,8 +1248,8 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
         g1.nx = g.nsplit;  // the min/max pass has no residual unit
         g1.d_nx.set(static_cast<uint32_t>(g.nsplit));
         // ... and keeps no logits, unless the table takes two passes (partial logits wait in the slots)
-        g1.cap = Lay<BITS, HPB, false, NT, F16K>::KPASS > 1 ? p.cap : 0;
-        const int lds_mm = Lay<BITS, HPB, false, NT, F16K>::lds_bytes(g1.cap);
+        g1.cap = (Lay<BITS, HPB, false, NT, REGL>::KPASS > 1 && REGL == 0) ? p.cap : 0;
+        const int lds_mm = Lay<BITS, HPB, false, NT, REGL>::lds_bytes(g1.cap);
         hipLaunchKernelGGL(kmm, dim3(units * g.nsplit), dim3(NT), lds_mm, st, g1);
         CQ_LAUNCH_CHECK();
     }
@@ -1300,9 +1267,9 @@ template <typename DT, bool VTOK>
 static int dispatch(const DecodeGeom& g, const Plan& p, int bits, hipStream_t st) {
     if (bits == 1) {
         if constexpr (!VTOK) {
-            if (p.hpb == 4 && p.nt == 512) return launch<1, 4, DT, false, 512, true>(g, p, st);
-            if (p.hpb == 4 && p.f16) return launch<1, 4, DT, false, 1024, true>(g, p, st);
-            if (p.hpb == 2 && p.nt == 512) return launch<1, 2, DT, false, 512, false>(g, p, st);
+            if (p.hpb == 4 && p.nt == 512) return launch<1, 4, DT, false, 512, kRegPair>(g, p, st);
+            if (p.hpb == 4 && p.regl) return launch<1, 4, DT, false, 1024, kRegLong>(g, p, st);
+            if (p.hpb == 2 && p.nt == 512) return launch<1, 2, DT, false, 512, 0>(g, p, st);
         }
         if (p.hpb == 4) return launch<1, 4, DT, VTOK>(g, p, st);
         if (p.hpb == 2) return launch<1, 2, DT, VTOK>(g, p, st);
@@ -1336,7 +1303,7 @@ int cq_decode_attn_plan(const cq_decode_args* args, cq_decode_plan* plan) {
     plan->chunk_tokens = args->T > 0 ? p.chunk : 0;
     plan->launches = p.nsplit > 1 ? 3 : 1;
     plan->lds_bytes = p.lds;
-    plan->f16_logits = p.f16;
+    plan->register_logits = p.regl;
     return CQ_OK;
 }
 

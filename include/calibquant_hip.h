@@ -195,7 +195,8 @@ typedef struct cq_decode_plan {
     int chunk_tokens;     /* packed tokens per chunk */
     int launches;         /* 1 or 3 */
     int lds_bytes;        /* dynamic LDS of the main launch */
-    int f16_logits;       /* non-zero: K table entries, look-up sums and waiting logits are packed fp16 */
+    int register_logits;  /* > 0: a thread keeps the logits of up to this many of its tokens in registers (fp32)
+                           * and the token slots in LDS hold only exp(.) as fp16; 0: fp32 logits wait in the slots */
 } cq_decode_plan;
 int cq_decode_attn_plan(const cq_decode_args* args, cq_decode_plan* plan);
 

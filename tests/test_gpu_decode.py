@@ -213,15 +213,15 @@ def test_decode_attn_full_batch_properties(ops):
 
 PAIRED = [
     # reps, Hq, Hkv, T, R, S, dtype, mask, calibrate — more than 256 units of work, a unit's layout within half the LDS:
-    # the launch uses 512-thread workgroups, two per compute unit (four heads per unit: packed-fp16 logits)
+    # the launch uses 512-thread workgroups, two per compute unit (four heads per unit: logits kept in registers, K table in two passes)
     (20, 32, 8, 777, 60, 41, "bf16", False, True),
     (20, 32, 8, 3328, 128, 0, "fp16", False, True),
     (20, 32, 8, 2100, 70, 5, "bf16", True, True),       # two blocks of staged value rows, mask
     (20, 32, 8, 300, 0, 0, "fp16", False, False),
-    (20, 16, 8, 1500, 130, 3, "bf16", True, True),      # two heads per unit: fp32 logits
+    (20, 16, 8, 1500, 130, 3, "bf16", True, True),      # two heads per unit: logits wait in the token slots
     (17, 48, 8, 1000, 33, 0, "fp16", False, True),      # six q heads per kv head: three units of two heads
     (20, 32, 8, 0, 200, 0, "bf16", False, True),        # window only
-    (12, 32, 8, 5000, 64, 0, "bf16", False, True),      # 192 units, T beyond the fp32 layout: one launch, packed-fp16 logits
+    (12, 32, 8, 5000, 64, 0, "bf16", False, True),      # 192 units, T beyond the layout with logits in the slots: one launch, logits in registers
     (8, 48, 8, 5000, 64, 3, "fp16", False, True),       # six q heads per kv head: two units of four heads, the second half padding
     (4, 32, 8, 9000, 100, 7, "bf16", False, True),      # chunked: 64 units x 8 chunks, min/max launch + merge
     (4, 32, 8, 9000, 0, 0, "fp16", True, True),
@@ -249,6 +249,31 @@ def test_decode_attn_paired_workgroups(ops, case):
     torch.cuda.synchronize()
     assert torch.equal(out, out[:2].repeat(reps, 1, 1))
     _check(to_np(out[:2]), _oracle(c, S, 1, mask=mask, calibrate_logits=calibrate))
+
+
+@pytest.mark.parametrize("mult, qscale", [(100.0, 1.0), (30.0, 3.0)])
+def test_decode_attn_paired_workgroups_large_logits(ops, mult, qscale):
+    """Key outlier channels x100 / queries x3: logits of magnitude 50-300 and a peaked softmax.  The
+    512-thread launch keeps its logits in fp32 (a 16-bit logit would be off by 2-4e-2 here)."""
+    from tests.util import CLIPS
+    reps, Hq, Hkv, T, R, D = 20, 32, 8, 3328, 128, 128
+    rng = np.random.default_rng(5)
+    k = rng.standard_normal((2, T, Hkv, D), dtype=np.float32)
+    v = rng.standard_normal((2, T, Hkv, D), dtype=np.float32)
+    for h in range(Hkv):
+        k[:, :, h, rng.permutation(D)[:4]] *= mult
+    k, v = O.round_to(k, "bf16"), O.round_to(v, "bf16")
+    ck, sk, zk = O.quantize_pack(k, 1, CLIPS[1][0], "bf16")
+    cv, sv, zv = O.quantize_pack(v, 1, CLIPS[1][1], "bf16")
+    c = dict(q=O.round_to(qscale * rng.standard_normal((2, Hq, D), dtype=np.float32), "bf16"), ck=ck, cv=cv, sk=sk, zk=zk,
+             sv=sv, zv=zv, kr=O.round_to(rng.standard_normal((2, Hkv, R, D), dtype=np.float32), "bf16"),
+             vr=O.round_to(rng.standard_normal((2, Hkv, R, D), dtype=np.float32), "bf16"))
+    g = case_to_gpu(c, "bf16")
+    rep = {n: torch.cat([t] * reps, 0) for n, t in g.items()}
+    out = ops.decode_attn(rep["q"], rep["ck"], rep["cv"], rep["sk"], rep["zk"], rep["sv"], rep["zv"], rep["kr"], rep["vr"])
+    torch.cuda.synchronize()
+    assert torch.equal(out, out[:2].repeat(reps, 1, 1))
+    _check(to_np(out[:2]), _oracle(c, 0, 1))
 
 
 def test_decode_attn_paired_workgroups_row_count_on_device(ops):

@@ -28,7 +28,7 @@ def test_library_loads_and_exports_every_declared_symbol():
 def test_decode_launch_plan_is_a_function_of_the_shape():
     """`cq_decode_attn_plan` (host only): which launch a shape gets.  Two 512-thread workgroups per compute
     unit need a layout within half of the 160 KB LDS and more units of work than the 256 compute units;
-    packed-fp16 logits only at 1 bit with four heads per unit; chunked shapes take three launches."""
+    logits kept in registers only at 1 bit with four heads per unit; chunked shapes take three launches."""
     from calibquant_amd import _lib
     lib = _lib.load()
 
@@ -40,20 +40,20 @@ def test_decode_launch_plan_is_a_function_of_the_shape():
         return {n: getattr(p, n) for n, _ in p._fields_}
 
     bench = plan(64, 32, 8, 3328, 128)
-    assert (bench["threads"], bench["heads_per_unit"], bench["launches"], bench["f16_logits"]) == (512, 4, 1, 1)
+    assert (bench["threads"], bench["heads_per_unit"], bench["launches"], bench["register_logits"]) == (512, 4, 1, 8)
     assert bench["lds_bytes"] <= 80 * 1024 and bench["chunk_tokens"] == 3328
     small = plan(32, 32, 8, 3328, 128)                       # 256 units: one 1024-thread workgroup per compute unit
-    assert (small["threads"], small["f16_logits"], small["launches"]) == (1024, 0, 1)
+    assert (small["threads"], small["register_logits"], small["launches"]) == (1024, 0, 1)
     assert plan(64, 32, 8, 3328, 128, bits=2)["threads"] == 1024
     assert plan(64, 32, 8, 3328, 128, v_mode=1)["threads"] == 1024
     assert plan(64, 32, 8, 3328, 128, force_splits=2) == dict(plan(64, 32, 8, 3328, 128, force_splits=2), threads=1024, launches=3)
     two = plan(128, 16, 8, 3328, 128)                        # two heads per unit: paired, fp32 logits
-    assert (two["threads"], two["heads_per_unit"], two["f16_logits"]) == (512, 2, 0)
+    assert (two["threads"], two["heads_per_unit"], two["register_logits"]) == (512, 2, 0)
     long = plan(8, 32, 8, 32768, 0)                          # chunked: the chunks are the units
     assert long["launches"] == 3 and long["threads"] == 512 and long["chunks"] * long["chunk_tokens"] >= 32768
     assert long["lds_bytes"] <= 80 * 1024
     big = plan(16, 48, 8, 9984, 64)     # six heads per kv head: two units of four (the second half padding); one launch
-    assert (big["threads"], big["heads_per_unit"], big["launches"], big["f16_logits"]) == (1024, 4, 1, 1)   # needs packed-fp16 logits
+    assert (big["threads"], big["heads_per_unit"], big["launches"], big["register_logits"]) == (1024, 4, 1, 10)   # logits in registers
     assert big["lds_bytes"] <= 160 * 1024
     assert plan(16, 48, 8, 9984, 64, v_mode=1)["heads_per_unit"] == 2
     a = _lib.DecodeArgs()
