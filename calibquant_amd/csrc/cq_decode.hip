@@ -1139,7 +1139,10 @@ static void plan_for(const cq_decode_args* a, Plan* p) {
         nsplit = need;
         if (a->force_splits > 0) {
             nsplit = a->force_splits > need ? a->force_splits : need;
-        } else if (units < 192) {
+        } else if (units < 192 && need > 1) {
+            // too few units to fill the device and T does not fit one unit anyway: more, smaller chunks.
+            // (A T that fits one unit is never chunked: the min/max launch's second pass over the packed
+            // K rows and the merge cost more than the idle compute units, at any batch size.)
             int64_t want = (512 + units - 1) / units;
             int64_t most = a->T / 1024 > 1 ? a->T / 1024 : 1;
             if (want > most) want = most;
