@@ -1212,6 +1212,22 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
         else if (G % 2 == 0) vtok ? plan_for<2, 2, true>(a, p) : plan_for<2, 2, false>(a, p);
         else vtok ? plan_for<2, 1, true>(a, p) : plan_for<2, 1, false>(a, p);
     }
+    // A handful of units leave most compute units idle, and a launch then lasts as long as one unit: fewer
+    // heads per unit make the units cheaper (18.8 / 15.5 / 14.2 us for four / two / one head at 3 328 + 128 tokens)
+    // and there are compute units for two or four times as many of them.
+    if (a->force_splits == 0 && p->nsplit == 1 && p->hpb == 4) {
+        const int64_t u4 = static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, 4);
+        const int h = u4 <= 32 ? 1 : (u4 <= 64 && G % 2 == 0) ? 2 : 4;
+        Plan q = *p;
+        if (a->bits == 1) {
+            if (h == 1) vtok ? plan_for<1, 1, true>(a, &q) : plan_for<1, 1, false>(a, &q);
+            if (h == 2) vtok ? plan_for<1, 2, true>(a, &q) : plan_for<1, 2, false>(a, &q);
+        } else {
+            if (h == 1) vtok ? plan_for<2, 1, true>(a, &q) : plan_for<2, 1, false>(a, &q);
+            if (h == 2) vtok ? plan_for<2, 2, true>(a, &q) : plan_for<2, 2, false>(a, &q);
+        }
+        if (q.nsplit == 1) *p = q;
+    }
     const int64_t blocks = static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, p->hpb) * p->nx;
     if (blocks > 0x7fffffff) return CQ_ERR_SHAPE;
     return CQ_OK;

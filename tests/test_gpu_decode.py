@@ -211,6 +211,45 @@ def test_decode_attn_full_batch_properties(ops):
     _check(to_np(out[:2]), _oracle(c, 0, 1))
 
 
+MID_BATCH = [
+    # reps, Hq, Hkv, T, R, S, bits, dtype, mask, token values — 65..256 units of four heads: one 1024-thread workgroup
+    # per unit, logits waiting in the token slots (smaller batches get fewer heads per unit)
+    (6, 32, 8, 3328, 128, 0, 1, "bf16", False, False),
+    (6, 32, 8, 777, 60, 41, 2, "fp16", True, False),     # 2 bits: K table in two passes, partial logits in the slots
+    (6, 32, 8, 1500, 33, 0, 1, "bf16", False, True),     # per-token values
+    (5, 48, 8, 1000, 70, 3, 2, "bf16", False, False),    # six q heads per kv head, padded four-head units
+    (6, 32, 8, 0, 150, 5, 1, "fp16", False, False),      # window only
+]
+
+
+@pytest.mark.parametrize("case", MID_BATCH, ids=lambda c: "-".join(str(x) for x in c))
+def test_decode_attn_mid_batch_four_heads_per_unit(ops, case):
+    reps, Hq, Hkv, T, R, S, bits, dtype, use_mask, token = case
+    c = make_case(2, Hq, Hkv, 128, max(T, 1), R, bits, dtype, seed=80 + T)
+    kw, okw = {}, {}
+    if token:
+        words, scale, mins = O.kivi_quantize_pack(np.transpose(c["v"], (0, 2, 1, 3)), 32, bits, dtype)
+        c["cv"], c["sv"], c["zv"] = words, scale, mins
+        kw["v_mode"], okw["v_token_group"] = "token", 32
+    if T == 0:
+        c["ck"], c["cv"] = c["ck"][:, :, :0], c["cv"][:, :, :0]
+    mask = None
+    if use_mask:
+        mask = np.where(np.random.default_rng(T).random((2, T + R)) < 0.15, -1e4, 0.0).astype(np.float32)
+    g = case_to_gpu(c, dtype)
+    rep = {k: torch.cat([v] * reps, 0) for k, v in g.items()}
+    m = None if mask is None else torch.from_numpy(mask).cuda().repeat(reps, 1)
+    args = [rep[k] if T else None for k in ("ck", "cv", "sk", "zk", "sv", "zv")]
+    call = ops.DecodeCall(rep["q"], *args, rep["kr"] if R else None, rep["vr"] if R else None,
+                          sprompt_len=S, bits=bits, mask=m, **kw)
+    plan = call.plan()
+    assert (plan["threads"], plan["heads_per_unit"], plan["launches"]) == (1024, 4, 1)
+    out = call.run()
+    torch.cuda.synchronize()
+    assert torch.equal(out, out[:2].repeat(reps, 1, 1))
+    _check(to_np(out[:2]), _oracle(c, S, bits, mask=mask, **okw))
+
+
 PAIRED = [
     # reps, Hq, Hkv, T, R, S, dtype, mask, calibrate — more than 256 units of work, a unit's layout within half the LDS:
     # the launch uses 512-thread workgroups, two per compute unit (four heads per unit: logits kept in registers, K table in two passes)
