@@ -245,7 +245,9 @@ __device__ __forceinline__ uint32_t pack_f16(float a, float b) {
 }
 
 template <int BITS, int HPB, typename DT, bool MINMAX_ONLY, bool VTOK = false, int NT = 1024, int REGL = 0>
-__global__ __launch_bounds__(NT) void decode_kernel(DecodeGeom g) {
+// (four waves per SIMD - at most 128 VGPRs - for either workgroup size: two 512-thread workgroups per compute
+// unit are only resident together within that)
+__global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
     using L = Lay<BITS, HPB, VTOK, NT, REGL>;
     using V = Vec<HPB>;
     constexpr int NB = L::NB;
