@@ -44,6 +44,7 @@ constexpr int kPF = 4;             // 16-byte loads kept in flight per thread an
 constexpr int kLdsMax = 160 * 1024;
 constexpr int kPairUnits = 256;    // compute units of the device this is laid out for
 constexpr int kRegPair = 8;        // rounds of logits a thread of a 512-thread workgroup keeps in registers (4 096 tokens)
+constexpr int kRegTwoBit = 4;      // ... of the 2-bit kernel with four heads per unit (4 096 tokens)
 constexpr int kRegLong = 10;       // ... of a 1024-thread workgroup that holds a long chunk in one launch (10 240 tokens)
 constexpr float kLog2e = 1.4426950408889634f;
 
@@ -1210,7 +1211,8 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
     } else {
         // four heads per unit need the two-pass K table; with per-token values their LDS layout
         // would not hold a 3 328-token chunk, so that mode keeps two heads per unit
-        if ((G % 4 == 0 || (G % 4 == 2 && G > 4)) && !vtok) plan_for<2, 4, false>(a, p);
+        // (the first pass's partial logits wait in registers, four tokens per thread: -3 % against the token slots)
+        if ((G % 4 == 0 || (G % 4 == 2 && G > 4)) && !vtok) plan_for<2, 4, false, 1024, kRegTwoBit>(a, p);
         else if (G % 2 == 0) vtok ? plan_for<2, 2, true>(a, p) : plan_for<2, 2, false>(a, p);
         else vtok ? plan_for<2, 1, true>(a, p) : plan_for<2, 1, false>(a, p);
     }
@@ -1297,7 +1299,7 @@ static int dispatch(const DecodeGeom& g, const Plan& p, int bits, hipStream_t st
         return launch<1, 1, DT, VTOK>(g, p, st);
     }
     if constexpr (!VTOK) {
-        if (p.hpb == 4) return launch<2, 4, DT, false>(g, p, st);
+        if (p.hpb == 4) return launch<2, 4, DT, false, 1024, kRegTwoBit>(g, p, st);
     }
     if (p.hpb == 2) return launch<2, 2, DT, VTOK>(g, p, st);
     return launch<2, 1, DT, VTOK>(g, p, st);
