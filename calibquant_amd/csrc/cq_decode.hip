@@ -101,15 +101,15 @@ template <int BITS, int HPB, bool VTOK = false, int NT_ = 1024, int REGL = 0> st
     static constexpr int ESZH = HW * 4;             // bytes per packed-fp16 table entry
     // The byte-indexed K table covers NBP byte positions at a time: all of them when that fits the
     // table's share of the LDS (64 KB; 32 KB for a 512-thread workgroup), else half of them in each of
-    // two passes over the chunk's rows, the first pass's partial logits waiting in the token slots or,
-    // with REGL, in registers.
+    // two (or a quarter in each of four) passes over the chunk's rows, the earlier passes' partial logits
+    // waiting in the token slots or, with REGL, in registers.
     static constexpr int KTMAX = (NT_ == 512 ? 32 : 64) * 1024;
-    static constexpr int KPASS = (NB * 256 * ESZ > KTMAX) ? 2 : 1;
+    static constexpr int KPASS = (NB * 256 * ESZ > 2 * KTMAX) ? 4 : (NB * 256 * ESZ > KTMAX) ? 2 : 1;
     static constexpr int NBP = NB / KPASS;          // byte positions per pass
     static constexpr int WPP = NBP / 4;             // 32-bit words of a row per pass
     static constexpr int PCS = (WPP + 3) / 4;       // 16-byte pieces of a row a pass looks at
     static constexpr int KT = NBP * 256 * ESZ;      // K table bytes
-    static_assert(NB * 256 * ESZ <= 2 * KTMAX, "at most two table passes");
+    static_assert(NB * 256 * ESZ <= 4 * KTMAX, "at most four table passes");
     static_assert(!(REGL > 0 && VTOK), "logits in registers: per-channel values only");
     static constexpr int SLOT = VTOK ? 16 : (REGL > 0 ? ESZH : ESZ);   // bytes per token slot: logits, later e (+ 4 group scales)
     static constexpr int NGRP = VTOK ? kD / 32 : 1; // channel groups with tables of their own
@@ -607,9 +607,15 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             }
         };
         k_pass(std::integral_constant<int, 0>{});
-        if constexpr (L::KPASS == 2) {
-            __syncthreads();   // every wave is done with the first pass's table
+        if constexpr (L::KPASS >= 2) {
+            __syncthreads();   // every wave is done with the previous pass's table
             k_pass(std::integral_constant<int, 1>{});
+        }
+        if constexpr (L::KPASS == 4) {
+            __syncthreads();
+            k_pass(std::integral_constant<int, 2>{});
+            __syncthreads();
+            k_pass(std::integral_constant<int, 3>{});
         }
     }
     if (n > 0) {   // one reduction for both: max of (-min, max)
@@ -1212,7 +1218,18 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
         // four heads per unit need the two-pass K table; with per-token values their LDS layout
         // would not hold a 3 328-token chunk, so that mode keeps two heads per unit
         // (the first pass's partial logits wait in registers, four tokens per thread: -3 % against the token slots)
-        if ((G % 4 == 0 || (G % 4 == 2 && G > 4)) && !vtok) plan_for<2, 4, false, 1024, kRegTwoBit>(a, p);
+        if ((G % 4 == 0 || (G % 4 == 2 && G > 4)) && !vtok) {
+            plan_for<2, 4, false, 1024, kRegTwoBit>(a, p);
+            // more units than compute units: two 512-thread workgroups per compute unit (K table in four passes)
+            const int64_t units = static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, 4);
+            if (a->force_splits == 0) {
+                Plan q;
+                plan_for<2, 4, false, 512, kRegPair>(a, &q);
+                const bool single = p->nsplit == 1 && q.nsplit == 1 && units > kPairUnits;
+                const bool chunked = p->nsplit > 1 && q.nsplit > 1 && units * q.nsplit > kPairUnits;
+                if ((single || chunked) && q.lds <= kLdsMax / 2) *p = q;
+            }
+        }
         else if (G % 2 == 0) vtok ? plan_for<2, 2, true>(a, p) : plan_for<2, 2, false>(a, p);
         else vtok ? plan_for<2, 1, true>(a, p) : plan_for<2, 1, false>(a, p);
     }
@@ -1299,6 +1316,7 @@ static int dispatch(const DecodeGeom& g, const Plan& p, int bits, hipStream_t st
         return launch<1, 1, DT, VTOK>(g, p, st);
     }
     if constexpr (!VTOK) {
+        if (p.hpb == 4 && p.nt == 512) return launch<2, 4, DT, false, 512, kRegPair>(g, p, st);
         if (p.hpb == 4) return launch<2, 4, DT, false, 1024, kRegTwoBit>(g, p, st);
     }
     if (p.hpb == 2) return launch<2, 2, DT, VTOK>(g, p, st);

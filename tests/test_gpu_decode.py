@@ -267,6 +267,34 @@ PAIRED = [
 ]
 
 
+PAIRED_2BIT = [
+    # reps, Hq, Hkv, T, R, S, dtype, mask — 2 bits, more than 256 four-head units: 512-thread workgroups, K table in four passes
+    (20, 32, 8, 3328, 128, 0, "bf16", False),
+    (20, 32, 8, 777, 60, 41, "fp16", True),
+    (17, 48, 8, 2100, 33, 0, "bf16", False),     # padded four-head units, two blocks of staged value rows
+    (4, 32, 8, 9000, 100, 7, "bf16", False),     # chunked
+]
+
+
+@pytest.mark.parametrize("case", PAIRED_2BIT, ids=lambda c: "-".join(str(x) for x in c))
+def test_decode_attn_paired_workgroups_two_bits(ops, case):
+    reps, Hq, Hkv, T, R, S, dtype, use_mask = case
+    c = make_case(2, Hq, Hkv, 128, T, R, 2, dtype, seed=90 + T, outlier_kind="x10" if T % 2 else "student")
+    mask = None
+    if use_mask:
+        mask = np.where(np.random.default_rng(T).random((2, T + R)) < 0.15, -1e4, 0.0).astype(np.float32)
+    g = case_to_gpu(c, dtype)
+    rep = {k: torch.cat([v] * reps, 0) for k, v in g.items()}
+    m = None if mask is None else torch.from_numpy(mask).cuda().repeat(reps, 1)
+    call = ops.DecodeCall(rep["q"], rep["ck"], rep["cv"], rep["sk"], rep["zk"], rep["sv"], rep["zv"], rep["kr"], rep["vr"],
+                          sprompt_len=S, bits=2, mask=m)
+    assert call.plan()["threads"] == 512
+    out = call.run()
+    torch.cuda.synchronize()
+    assert torch.equal(out, out[:2].repeat(reps, 1, 1))
+    _check(to_np(out[:2]), _oracle(c, S, 2, mask=mask))
+
+
 @pytest.mark.parametrize("case", PAIRED, ids=lambda c: "-".join(str(x) for x in c))
 def test_decode_attn_paired_workgroups(ops, case):
     """Batches with more units of work than compute units: every batch row is an independent problem, so

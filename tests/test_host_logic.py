@@ -44,7 +44,9 @@ def test_decode_launch_plan_is_a_function_of_the_shape():
     assert bench["lds_bytes"] <= 80 * 1024 and bench["chunk_tokens"] == 3328
     small = plan(32, 32, 8, 3328, 128)                       # 256 units: one 1024-thread workgroup per compute unit
     assert (small["threads"], small["register_logits"], small["launches"]) == (1024, 0, 1)
-    assert plan(64, 32, 8, 3328, 128, bits=2)["threads"] == 1024
+    two_bit = plan(64, 32, 8, 3328, 128, bits=2)            # 2 bits: paired as well, K table in four passes
+    assert (two_bit["threads"], two_bit["register_logits"]) == (512, 8) and two_bit["lds_bytes"] <= 80 * 1024
+    assert plan(32, 32, 8, 3328, 128, bits=2)["threads"] == 1024
     assert plan(64, 32, 8, 3328, 128, v_mode=1)["threads"] == 1024
     assert plan(64, 32, 8, 3328, 128, force_splits=2) == dict(plan(64, 32, 8, 3328, 128, force_splits=2), threads=1024, launches=3)
     two = plan(128, 16, 8, 3328, 128)                        # two heads per unit: paired, fp32 logits
