@@ -188,6 +188,18 @@ def side_legs(torch, ops, shape, bits, sets):
     res["per_token_values"] = {"quantize_pack_token_us": round(ms_t * 1e3, 1), "decode_us_layer": round(ms_d * 1e3, 2),
                                "algorithmic_bytes": nb, "achieved_GBps": round(nb / ms_d / 1e6, 1),
                                "note": "one buffer set (codes may be served from the Infinity Cache)"}
+    del words, vsc, vmn, call
+    # the other bit width of the same layer shape (BASELINE's layer configuration names b = 1 and b = 2)
+    ob = 2 if bits == 1 else 1
+    osets = build_sets(torch, ops, shape, ob, 2, 4321)
+    ocalls = [ops.DecodeCall(x["q"], x["ck"], x["cv"], x["sk"], x["zk"], x["sv"], x["zv"], x["kr"], x["vr"],
+                             sprompt_len=S, bits=ob) for x in osets]
+    ms_o = time_calls(torch, ocalls, 100, 10)
+    nbo = algorithmic_bytes(B, Hq, Hkv, D, T, R, ob)
+    res[f"decode_{ob}bit"] = {"us_layer": round(ms_o * 1e3, 2), "algorithmic_bytes": nbo,
+                              "achieved_GBps": round(nbo / ms_o / 1e6, 1),
+                              "frac_of_hbm_peak": round(nbo / ms_o / 1e6 / HBM_PEAK_GBPS, 4),
+                              "launch_plan": ocalls[0].plan(), "note": "two buffer sets"}
     return res
 
 
