@@ -63,6 +63,38 @@ def test_decode_launch_plan_is_a_function_of_the_shape():
     assert lib.cq_decode_attn_plan(ctypes.byref(a), ctypes.byref(_lib.DecodePlan())) < 0   # all-zero arguments
 
 
+def test_decode_launch_plan_invariants_over_random_shapes():
+    """Whatever the shape, the plan stays inside what the kernels assume: LDS within the device's 160 KB (half of
+    it for a 512-thread workgroup), chunks that cover T, register-resident logits only for chunks that fit the
+    rounds a thread keeps, three launches and a workspace exactly when T is chunked."""
+    from calibquant_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(11)
+    for _ in range(3000):
+        Hkv = int(rng.choice([1, 2, 4, 8, 16]))
+        G = int(rng.choice([1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 16]))
+        a = _lib.DecodeArgs()
+        a.dtype, a.D, a.Hkv, a.Hq = int(rng.integers(0, 2)), 128, Hkv, Hkv * G
+        a.B = int(rng.choice([1, 2, 3, 8, 16, 31, 32, 33, 64, 100, 256, 1000]))
+        a.T = int(rng.choice([0, 1, 63, 64, 65, 1000, 3328, 3392, 4096, 4097, 4288, 5000, 9984, 10240, 10241, 32768, 100000]))
+        a.R = int(rng.choice([0, 1, 64, 128, 129, 1000])) if a.T else int(rng.choice([1, 64, 500]))
+        a.bits = int(rng.integers(1, 3))
+        a.v_mode = int(rng.integers(0, 2))
+        a.force_splits = int(rng.choice([0, 0, 0, 1, 2, 7]))
+        p = _lib.DecodePlan()
+        assert lib.cq_decode_attn_plan(ctypes.byref(a), ctypes.byref(p)) == 0
+        shape = (a.B, a.Hq, a.Hkv, a.T, a.R, a.bits, a.v_mode, a.force_splits)
+        assert p.threads in (512, 1024) and p.heads_per_unit in (1, 2, 4), shape
+        assert 0 < p.lds_bytes <= (80 if p.threads == 512 else 160) * 1024, shape
+        assert p.chunks >= 1 and p.chunks * p.chunk_tokens >= a.T, shape
+        assert p.chunk_tokens % 64 == 0, shape
+        assert p.register_logits == 0 or p.chunk_tokens <= p.register_logits * p.threads, shape
+        assert p.launches == (3 if p.chunks > 1 else 1), shape
+        assert (lib.cq_decode_attn_workspace(ctypes.byref(a)) > 0) == (p.chunks > 1), shape
+        if a.v_mode == 1:
+            assert p.threads == 1024 and p.register_logits == 0, shape
+
+
 def test_c_abi_rejects_bad_arguments_without_touching_the_gpu():
     """Validation happens before any launch, so these calls are safe without a device."""
     from calibquant_amd import _lib
