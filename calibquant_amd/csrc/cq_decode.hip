@@ -1186,9 +1186,9 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
     if (a->v_mode != CQ_V_PER_CHANNEL && a->v_mode != CQ_V_PER_TOKEN) return CQ_ERR_UNSUPPORTED;
     const bool vtok = a->v_mode == CQ_V_PER_TOKEN;
     if (a->bits == 1) {
-        // G = 6, 10, ...: units of four heads with the last one half padding (two units per kv head at
-        // G = 6) do less work than units of two heads (three of them, each walking all the packed rows)
-        const bool pad4 = G % 4 == 2 && G > 4 && !vtok;
+        // G = 3, 5, 6, 7, ...: units of four heads with the last one partly padding (two units per kv head at
+        // G = 6) do less work than units of two heads or one (three or six of them, each walking all the packed rows)
+        const bool pad4 = G % 4 != 0 && G > 2 && !vtok;
         if (G % 4 == 0 || pad4) vtok ? plan_for<1, 4, true>(a, p) : plan_for<1, 4, false>(a, p);
         else if (G % 2 == 0) vtok ? plan_for<1, 2, true>(a, p) : plan_for<1, 2, false>(a, p);
         else vtok ? plan_for<1, 1, true>(a, p) : plan_for<1, 1, false>(a, p);
@@ -1218,7 +1218,7 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
         // four heads per unit need the two-pass K table; with per-token values their LDS layout
         // would not hold a 3 328-token chunk, so that mode keeps two heads per unit
         // (the first pass's partial logits wait in registers, four tokens per thread: -3 % against the token slots)
-        if ((G % 4 == 0 || (G % 4 == 2 && G > 4)) && !vtok) {
+        if ((G % 4 == 0 || G > 2) && !vtok) {
             plan_for<2, 4, false, 1024, kRegTwoBit>(a, p);
             // more units than compute units: two 512-thread workgroups per compute unit (K table in four passes)
             const int64_t units = static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, 4);

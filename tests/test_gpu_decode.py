@@ -219,6 +219,9 @@ MID_BATCH = [
     (6, 32, 8, 1500, 33, 0, 1, "bf16", False, True),     # per-token values
     (5, 48, 8, 1000, 70, 3, 2, "bf16", False, False),    # six q heads per kv head, padded four-head units
     (6, 32, 8, 0, 150, 5, 1, "fp16", False, False),      # window only
+    (6, 56, 8, 900, 40, 0, 1, "bf16", False, False),     # seven q heads per kv head: units of 4 + 3
+    (8, 40, 8, 600, 70, 9, 2, "fp16", True, False),      # five: units of 4 + 1
+    (10, 24, 8, 700, 20, 0, 1, "bf16", False, False),    # three: one unit of four heads, one of them padding
 ]
 
 
@@ -260,6 +263,7 @@ PAIRED = [
     (20, 16, 8, 1500, 130, 3, "bf16", True, True),      # two heads per unit: logits wait in the token slots
     (17, 48, 8, 1000, 33, 0, "fp16", False, True),      # six q heads per kv head: three units of two heads
     (20, 32, 8, 0, 200, 0, "bf16", False, True),        # window only
+    (12, 56, 8, 1200, 64, 2, "fp16", False, True),      # seven q heads per kv head: padded four-head units, paired
     (12, 32, 8, 5000, 64, 0, "bf16", False, True),      # 192 units, T beyond the layout with logits in the slots: one launch, logits in registers
     (8, 48, 8, 5000, 64, 3, "fp16", False, True),       # six q heads per kv head: two units of four heads, the second half padding
     (4, 32, 8, 9000, 100, 7, "bf16", False, True),      # chunked: 64 units x 8 chunks, min/max launch + merge
