@@ -1188,7 +1188,7 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
     if (a->bits == 1) {
         // G = 3, 5, 6, 7, ...: units of four heads with the last one partly padding (two units per kv head at
         // G = 6) do less work than units of two heads or one (three or six of them, each walking all the packed rows)
-        const bool pad4 = G % 4 != 0 && G > 2 && !vtok;
+        const bool pad4 = G % 4 != 0 && G > 2;
         if (G % 4 == 0 || pad4) vtok ? plan_for<1, 4, true>(a, p) : plan_for<1, 4, false>(a, p);
         else if (G % 2 == 0) vtok ? plan_for<1, 2, true>(a, p) : plan_for<1, 2, false>(a, p);
         else vtok ? plan_for<1, 1, true>(a, p) : plan_for<1, 1, false>(a, p);
@@ -1230,7 +1230,7 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
                 if ((single || chunked) && q.lds <= kLdsMax / 2) *p = q;
             }
         }
-        else if (G % 2 == 0) vtok ? plan_for<2, 2, true>(a, p) : plan_for<2, 2, false>(a, p);
+        else if (G >= 2) vtok ? plan_for<2, 2, true>(a, p) : plan_for<2, 2, false>(a, p);   // (per-token values: two heads per unit, padded for odd G)
         else vtok ? plan_for<2, 1, true>(a, p) : plan_for<2, 1, false>(a, p);
     }
     // A handful of units leave most compute units idle, and a launch then lasts as long as one unit: fewer

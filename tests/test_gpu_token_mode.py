@@ -45,6 +45,7 @@ CASES = [
     (2, 32, 8, 777, 60, 41),       # ragged T, system prompt rows
     (1, 48, 8, 1000, 33, 0),       # six q heads per kv head
     (1, 8, 8, 130, 0, 0),          # one q head per kv head, no residual
+    (12, 56, 8, 700, 20, 3),       # seven q heads per kv head: padded units (four heads at 1 bit, two at 2 bits)
 ]
 
 

@@ -57,7 +57,8 @@ def test_decode_launch_plan_is_a_function_of_the_shape():
     big = plan(16, 48, 8, 9984, 64)     # six heads per kv head: two units of four (the second half padding); one launch
     assert (big["threads"], big["heads_per_unit"], big["launches"], big["register_logits"]) == (1024, 4, 1, 10)   # logits in registers
     assert big["lds_bytes"] <= 160 * 1024
-    assert plan(16, 48, 8, 9984, 64, v_mode=1)["heads_per_unit"] == 2
+    tok = plan(16, 48, 8, 9984, 64, v_mode=1)               # per-token values: padded four-head units too, chunked (16-byte slots)
+    assert (tok["heads_per_unit"], tok["threads"], tok["register_logits"]) == (4, 1024, 0) and tok["launches"] == 3
     a = _lib.DecodeArgs()
     assert lib.cq_decode_attn_plan(ctypes.byref(a), None) < 0
     assert lib.cq_decode_attn_plan(ctypes.byref(a), ctypes.byref(_lib.DecodePlan())) < 0   # all-zero arguments
