@@ -8,7 +8,7 @@ batch 64, 32 query / 8 KV heads, head_dim 128, 3 328 packed image tokens plus a
 region; the call rotates over several distinct buffer sets (> 256 MB in total)
 so the packed codes are not served from the Infinity Cache.
 
-Prints ONE JSON line (see README / DESIGN for the fields).  `value` is the
+Prints ONE JSON line.  `value` is the
 average duration of one layer call in microseconds; `roofline` prices the
 algorithmic bytes of that call against the 8 TB/s HBM peak; `cpu_baseline` is
 the C port of the oracle timed on this host's cores on a bounded sample.
