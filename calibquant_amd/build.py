@@ -25,6 +25,11 @@ FLAGS = [
     "-Wall", "-Wno-unused-command-line-argument",
     "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
 ]
+# per-source additions.  The decode kernels are bound by vector-instruction issue: the
+# ILP-first machine scheduler measures 1-3 % faster there (same register counts, no scratch).
+EXTRA_FLAGS = {
+    "cq_decode.hip": ["-mllvm", "-amdgpu-sched-strategy=max-ilp"],
+}
 
 
 def build(verbose: bool = True, jobs: int = 4) -> str:
@@ -33,7 +38,7 @@ def build(verbose: bool = True, jobs: int = 4) -> str:
     for src in SOURCES:
         obj = os.path.join(LIBDIR, src.replace(".hip", ".o"))
         objs.append(obj)
-        cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [HIPCC, *FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
