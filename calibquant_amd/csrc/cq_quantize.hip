@@ -348,40 +348,65 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
     // during the emit and its min / max pass starts without a wait.
     const int nslice = static_cast<int>((static_cast<int64_t>(g.B) * g.H + 7) / 8) * 32;
     const int64_t nbh = static_cast<int64_t>(g.B) * g.H;
-    auto slice_base = [&](int vb) -> const uint16_t* {   // slices past the last (batch, head) alias the last one
+    // The slice's base is the same for the whole workgroup and a row's piece sits at a 32-bit byte
+    // offset from it (the host checks T * row stride < 2^24 bytes): a load takes its address as
+    // scalar base + vector offset, one 24-bit multiply-add per row.
+    auto slice_base = [&](int vb) -> const unsigned char* {   // slices past the last (batch, head) alias the last one
         const int quarter = (vb >> 3) & 3;
         const uint32_t bh = static_cast<uint32_t>(min(static_cast<int64_t>(vb >> 5) * 8 + (vb & 7), nbh - 1));
         const uint32_t b = g.dH.quot(bh), h = bh - b * g.dH.div;   // B * H < 2^31 on this path
-        return x + static_cast<int64_t>(b) * g.sb + static_cast<int64_t>(h) * g.sh + quarter * 32 + q4 * 8;
+        return reinterpret_cast<const unsigned char*>(x + static_cast<int64_t>(b) * g.sb + static_cast<int64_t>(h) * g.sh + quarter * 32);
+    };
+    const uint32_t st_bytes = static_cast<uint32_t>(g.st) * 2u, q_bytes = static_cast<uint32_t>(q4) * 16u;
+    auto row_offset = [&](int t) -> uint32_t {   // byte offset of the thread's piece of row min(t, T - 1)
+        return static_cast<uint32_t>(__umul24(static_cast<uint32_t>(min(t, g.T - 1)), st_bytes)) + q_bytes;
     };
     typedef uint32_t U4 __attribute__((ext_vector_type(4)));
     U4 v[NR];
     {
-        const uint16_t* base = slice_base(blockIdx.x);
+        const unsigned char* base = slice_base(blockIdx.x);
 #pragma unroll
-        for (int i = 0; i < NR; ++i) {   // rows past T re-read row T-1: min / max unchanged, never written
-            const int t = min(i * (kFThreads / 4) + row, g.T - 1);
-            v[i] = *reinterpret_cast<const U4*>(base + t * g.st);
-        }
+        for (int i = 0; i < NR; ++i)   // rows past T re-read row T-1: min / max unchanged, never written
+            v[i] = *reinterpret_cast<const U4*>(base + row_offset(i * (kFThreads / 4) + row));
     }
     for (int vb = blockIdx.x; vb < nslice; vb += gridDim.x) {
     const int quarter = (vb >> 3) & 3;
     const int64_t bh = static_cast<int64_t>(vb >> 5) * 8 + (vb & 7);
     const bool live = bh < nbh;                         // a padding slice computes and writes nothing
     const bool has_next = vb + static_cast<int>(gridDim.x) < nslice;
-    const uint16_t* next_base = slice_base(has_next ? vb + gridDim.x : vb);
+    const unsigned char* next_base = slice_base(has_next ? vb + gridDim.x : vb);
     int row_i = row;   // opaque per iteration: the row offsets below are recomputed, not kept in registers across the loop
     asm volatile("" : "+v"(row_i));
-    float mn[8], mx[8];
+    // Both storage types are sign-magnitude, so the extremes of a column follow from three packed
+    // 16-bit integer folds of the raw words, two elements per instruction and no unpacking: as
+    // signed integers the non-negative values are in value order (the signed maximum is the
+    // largest of them, if there is one); as unsigned integers the negative values lie above every
+    // non-negative one, in order of magnitude (the unsigned maximum is the most negative value,
+    // if there is one; the unsigned minimum is the smallest non-negative value, or with negatives
+    // only the one nearest to zero).  -0 counts as negative and orders below +0.
+    typedef short S2 __attribute__((ext_vector_type(2)));
+    typedef unsigned short US2 __attribute__((ext_vector_type(2)));
+    uint32_t k_smax[4], k_umin[4], k_umax[4];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) { mn[j] = INFINITY; mx[j] = -INFINITY; }
+    for (int w = 0; w < 4; ++w) { k_smax[w] = 0x80008000u; k_umin[w] = 0xffffffffu; k_umax[w] = 0u; }
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
-        float f[8];
-        unpack8<DT>(v[i], f);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) { mn[j] = fminf(mn[j], f[j]); mx[j] = fmaxf(mx[j], f[j]); }
-        __builtin_amdgcn_sched_barrier(0);   // one row at a time: unpacking all rows ahead would not fit the registers
+        for (int w = 0; w < 4; ++w) {
+            const uint32_t r = v[i][w];
+            k_smax[w] = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(S2, k_smax[w]), __builtin_bit_cast(S2, r)));
+            k_umin[w] = __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(US2, k_umin[w]), __builtin_bit_cast(US2, r)));
+            k_umax[w] = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(US2, k_umax[w]), __builtin_bit_cast(US2, r)));
+        }
+    }
+    float mn[8], mx[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int sh = 16 * (j & 1);
+        const uint32_t smax = (k_smax[j >> 1] >> sh) & 0xffffu, umin = (k_umin[j >> 1] >> sh) & 0xffffu,
+                       umax = (k_umax[j >> 1] >> sh) & 0xffffu;
+        mn[j] = Cvt<DT>::to_float((umax & 0x8000u) ? umax : umin);
+        mx[j] = Cvt<DT>::to_float((smax & 0x8000u) ? umin : smax);
     }
     // lanes l, l+4, l+8, l+12 of a row of 16 lanes hold the same channels: two rotations fold them
 #pragma unroll
@@ -467,16 +492,44 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
         float f[8];
         unpack8<DT>(v[i], f);
         uint32_t code[8];
+        if constexpr (BITS == 2) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            code[j] = (f[j] >= th[0][j]) ? 1u : 0u;
-            if constexpr (BITS == 2) code[j] += ((f[j] >= th[1][j]) ? 1u : 0u) + ((f[j] >= th[2][j]) ? 1u : 0u);
+            for (int j = 0; j < 8; ++j)
+                code[j] = ((f[j] >= th[0][j]) ? 1u : 0u) + ((f[j] >= th[1][j]) ? 1u : 0u) + ((f[j] >= th[2][j]) ? 1u : 0u);
         }
         uint8_t* o = codes + (min(bh, nbh - 1) * g.T + min(t, g.T - 1)) * nb + quarter * (nb / 4);
         if constexpr (BITS == 1) {
+            // The byte is built by eight add-with-carry steps, w = w + w + (f[j] >= th[j]): each
+            // comparison leaves its lane mask in a scalar register pair of its own and the add
+            // takes it as the carry-in (two instructions per element; a compare, a select and an
+            // OR otherwise).  The compares come first, so every mask is read at least two
+            // instructions after it is written, as this chip requires of a vector instruction
+            // that reads a scalar register written by another.
             uint32_t w = 0;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) w |= code[j] << (7 - j);
+            unsigned long long m0, m1, m2, m3, m4, m5, m6, m7;
+            asm volatile(
+                "v_cmp_le_f32_e64 %[m0], %[t0], %[f0]\n\t"
+                "v_cmp_le_f32_e64 %[m1], %[t1], %[f1]\n\t"
+                "v_cmp_le_f32_e64 %[m2], %[t2], %[f2]\n\t"
+                "v_cmp_le_f32_e64 %[m3], %[t3], %[f3]\n\t"
+                "v_cmp_le_f32_e64 %[m4], %[t4], %[f4]\n\t"
+                "v_cmp_le_f32_e64 %[m5], %[t5], %[f5]\n\t"
+                "v_cmp_le_f32_e64 %[m6], %[t6], %[f6]\n\t"
+                "v_cmp_le_f32_e64 %[m7], %[t7], %[f7]\n\t"
+                "v_addc_co_u32_e64 %[w], %[m0], %[w], %[w], %[m0]\n\t"
+                "v_addc_co_u32_e64 %[w], %[m1], %[w], %[w], %[m1]\n\t"
+                "v_addc_co_u32_e64 %[w], %[m2], %[w], %[w], %[m2]\n\t"
+                "v_addc_co_u32_e64 %[w], %[m3], %[w], %[w], %[m3]\n\t"
+                "v_addc_co_u32_e64 %[w], %[m4], %[w], %[w], %[m4]\n\t"
+                "v_addc_co_u32_e64 %[w], %[m5], %[w], %[w], %[m5]\n\t"
+                "v_addc_co_u32_e64 %[w], %[m6], %[w], %[w], %[m6]\n\t"
+                "v_addc_co_u32_e64 %[w], %[m7], %[w], %[w], %[m7]"
+                : [w] "+v"(w), [m0] "=&s"(m0), [m1] "=&s"(m1), [m2] "=&s"(m2), [m3] "=&s"(m3),
+                  [m4] "=&s"(m4), [m5] "=&s"(m5), [m6] "=&s"(m6), [m7] "=&s"(m7)
+                : [t0] "v"(th[0][0]), [t1] "v"(th[0][1]), [t2] "v"(th[0][2]), [t3] "v"(th[0][3]),
+                  [t4] "v"(th[0][4]), [t5] "v"(th[0][5]), [t6] "v"(th[0][6]), [t7] "v"(th[0][7]),
+                  [f0] "v"(f[0]), [f1] "v"(f[1]), [f2] "v"(f[2]), [f3] "v"(f[3]),
+                  [f4] "v"(f[4]), [f5] "v"(f[5]), [f6] "v"(f[6]), [f7] "v"(f[7]));
             w <<= 8 * q4;
             w |= static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(w), 0xB1, 0xf, 0xf, true));
             w |= static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(w), 0x4E, 0xf, 0xf, true));
@@ -489,7 +542,7 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
             if ((q4 & 1) == 0 && t < g.T && live) reinterpret_cast<uint32_t*>(o)[q4 >> 1] = half | (other << 16);
         }
         // the row is packed: its registers take the same row of the next slice
-        if (has_next) v[i] = *reinterpret_cast<const U4*>(next_base + min(t, g.T - 1) * g.st);
+        if (has_next) v[i] = *reinterpret_cast<const U4*>(next_base + row_offset(t));
     }
     }
 }
@@ -502,7 +555,8 @@ static int run_quant(const void* x, QuantGeom g, int bits, float clip, uint8_t* 
     uint16_t* sp = static_cast<uint16_t*>(scale);
     uint16_t* zp = static_cast<uint16_t*>(zero);
     if (!xq && g.D == 128 && g.T <= kFMaxT && (reinterpret_cast<uintptr_t>(codes) & 3u) == 0 &&
-        static_cast<int64_t>(g.B) * g.H < (static_cast<int64_t>(1) << 31)) {
+        static_cast<int64_t>(g.B) * g.H < (static_cast<int64_t>(1) << 31) &&
+        g.st > 0 && g.st * 2 < (1 << 24) && static_cast<int64_t>(g.T) * g.st * 2 < (static_cast<int64_t>(1) << 31)) {   // 32-bit row offsets
         // x fits a workgroup's registers slice by slice: one pass
         const int64_t bh8 = (static_cast<int64_t>(g.B) * g.H + 7) / 8;
         // persistent: at most one workgroup per compute unit and a multiple of 32 of them
