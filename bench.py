@@ -316,7 +316,7 @@ def model_leg(torch, batch=64, tiles=13, sys_len=41, text_len=23, new_tokens=128
             emb[ids == model.img_context_token_id] = vit.reshape(-1, emb.shape[-1])
             if patched:
                 for layer in lm.model.layers:
-                    layer.attention.image_token_num = T
+                    layer.attention.cq_image_token_num = T
             pos = torch.arange(N, device=dev)[None].expand(batch, N)
             logits, past = lm.forward_step(emb, pos, None)
             del emb, vit

@@ -14,7 +14,7 @@ CQ_BF16, CQ_FP16, CQ_FP32, CQ_I64, CQ_I32, CQ_U8 = range(6)
 
 SYMBOLS = (
     "cq_version", "cq_strerror", "cq_last_hip_error",
-    "cq_quantize_pack_workspace", "cq_quantize_pack", "cq_quant", "cq_encode",
+    "cq_quantize_pack_workspace", "cq_quantize_pack", "cq_quant", "cq_quant_tensor", "cq_encode",
     "cq_lut_vecmat_qk", "cq_lut_vecmat_pv",
     "cq_decode_attn_workspace", "cq_decode_attn", "cq_decode_attn_plan", "cq_rope_append", "cq_quantize_pack_token",
 )
@@ -76,9 +76,11 @@ def load() -> C.CDLL:
     lib.cq_quantize_pack.argtypes = qargs
     lib.cq_quant.restype = i
     lib.cq_quant.argtypes = qargs
+    lib.cq_quant_tensor.restype = i
+    lib.cq_quant_tensor.argtypes = qargs
     lib.cq_encode.restype = i
     lib.cq_encode.argtypes = [vp, i, i64, i, i, vp, vp]
-    vm = [vp, i, vp, i, vp, i64, i, i, i, vp, vp]
+    vm = [vp, i, i, vp, i, vp, i64, i, i, i, vp, vp]
     lib.cq_lut_vecmat_qk.restype = i
     lib.cq_lut_vecmat_qk.argtypes = vm
     lib.cq_lut_vecmat_pv.restype = i

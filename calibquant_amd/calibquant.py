@@ -36,18 +36,20 @@ def quant(x, bits, per_channel=False, scale=1, post_scale=False):
 
     x: (B, T, H, D) bf16 / fp16 GPU tensor (any strides with a contiguous last
     axis).  `per_channel=True` reduces over dim 1, one scale / zero-point per
-    (batch, head, channel); this is the only mode the attention path uses
-    (patch_internvl.py:181,187) and the only one implemented here.
+    (batch, head, channel), shaped (B, 1, H, D); this is the mode the attention
+    path uses (patch_internvl.py:181,187).  `per_channel=False` takes one
+    minimum and maximum over the whole tensor (calibquant.py:29-31); scale and
+    zero_point are then 0-d tensors.
     Returns `(x_q, scale, zero_point)` when `post_scale` is set, else
-    `(dequantised x, scale, zero_point)`; scale and zero_point are (B, 1, H, D).
+    `(dequantised x, scale, zero_point)`.
     Arithmetic rounds to x.dtype after every step, as the reference's chain of
     torch ops does."""
-    if not per_channel:
-        raise CalibQuantError("quant(per_channel=False) is not part of the decode path and is not implemented; "
-                              "the attention forward always passes per_channel=True")
     if bits not in (1, 2):
         raise CalibQuantError(f"quant: {bits}-bit codes are not supported (1 or 2)")
-    x_q, s, z = ops.quant_codes(x, int(bits), float(scale))
+    if per_channel:
+        x_q, s, z = ops.quant_codes(x, int(bits), float(scale))
+    else:
+        x_q, s, z = ops.quant_codes_tensor(x, int(bits), float(scale))
     if post_scale:
         return x_q, s, z
     return s * (x_q - z), s, z          # calibquant.py:38, same two torch ops

@@ -7,7 +7,7 @@ thread_local int g_last_hip_error = 0;
 
 extern "C" {
 
-int cq_version(void) { return 101; }   // 101: cq_decode_attn_plan
+int cq_version(void) { return 102; }   // 102: lut_len argument of the look-up vec-mats, cq_quant_tensor
 
 const char* cq_strerror(int status) {
     switch (status) {

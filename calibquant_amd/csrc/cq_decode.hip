@@ -42,7 +42,7 @@ namespace cq {
 constexpr int kD = 128;
 constexpr int kPF = 4;             // 16-byte loads kept in flight per thread and stream
 constexpr int kLdsMax = 160 * 1024;
-constexpr int kPairUnits = 256;    // compute units of the device this is laid out for
+constexpr int kDefaultUnits = 256; // compute units of a whole MI355X, assumed when no device can be asked
 constexpr int kRegPair = 8;        // rounds of logits a thread of a 512-thread workgroup keeps in registers (4 096 tokens)
 constexpr int kRegTwoBit = 4;      // ... of the 2-bit kernel with four heads per unit (4 096 tokens)
 constexpr int kRegLong = 10;       // ... of a 1024-thread workgroup that holds a long chunk in one launch (10 240 tokens)
@@ -1127,6 +1127,22 @@ __global__ void merge_kernel(const float* __restrict__ part, int nx, void* __res
     store_elem<DT>(out, row * kD + d, num / den);
 }
 
+// Compute units of the current device (a partitioned device reports its own share), asked once per
+// process; kDefaultUnits when there is no device to ask (a host that only plans).
+static int pair_units() {
+    static std::atomic<int> cached{0};
+    int n = cached.load(std::memory_order_relaxed);
+    if (n > 0) return n;
+    int dev = 0, cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cu < 1) {
+        (void)hipGetLastError();   // not an error of the caller's
+        cu = kDefaultUnits;
+    }
+    cached.store(cu, std::memory_order_relaxed);
+    return cu;
+}
+
 // head groups per kv head; the last one may be partly padding (its spare heads repeat its last query head
 // and write nothing)
 static inline int ngroups(int G, int hpb) { return (G + hpb - 1) / hpb; }
@@ -1176,6 +1192,7 @@ static void plan_for(const cq_decode_args* a, Plan* p) {
 
 static int make_plan(const cq_decode_args* a, Plan* p) {
     if (!a) return CQ_ERR_NULL;
+    const int kPairUnits = pair_units();
     if (a->dtype != CQ_BF16 && a->dtype != CQ_FP16) return CQ_ERR_DTYPE;
     if (a->bits != 1 && a->bits != 2) return CQ_ERR_UNSUPPORTED;
     if (a->D != kD) return CQ_ERR_UNSUPPORTED;

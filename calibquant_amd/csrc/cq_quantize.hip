@@ -31,6 +31,7 @@ struct QuantGeom {
     int64_t sb, st, sh;   // element strides of x
     int nchunk, chunk;    // token chunks
     FastDiv dT, dH;       // divisors T and H of a flat (b, h, t) row index (per-token quantiser)
+    int shared_stats;     // non-zero: one row of statistics / thresholds serves every (batch, head) (whole-tensor mode)
 };
 
 static inline int pick_chunks(int B, int T, int H) {
@@ -188,6 +189,79 @@ __global__ void stats_kernel(const float* __restrict__ part, QuantGeom g, float 
     o[(k - 1) * g.D] = t;
 }
 
+// Whole-tensor statistics (`per_channel=False`, calibquant.py:29-31: x.min() * scale, x.max() * scale):
+// one 1024-thread workgroup folds every chunk partial into a single (min, max), runs the same op chain
+// and threshold search as above, and writes one row of D identical statistics / thresholds that the
+// emit kernel reads for every (batch, head), plus the two scalars the caller gets back.
+template <typename DT>
+__global__ __launch_bounds__(kStatThreads) void tensor_stats_kernel(const float* __restrict__ part, int64_t npairs, int D,
+                                                                    float clip, float levels,
+                                                                    uint16_t* __restrict__ scale_row,
+                                                                    uint16_t* __restrict__ zero_row,
+                                                                    float* __restrict__ thr_row,
+                                                                    uint16_t* __restrict__ scale1,
+                                                                    uint16_t* __restrict__ zero1) {
+    __shared__ float smn[kStatThreads / kWave], smx[kStatThreads / kWave];
+    __shared__ float st[2 + 3];   // scale, zero-point, thresholds
+    const int tid = threadIdx.x;
+    float a = INFINITY, z = -INFINITY;
+    const int64_t n = npairs * 2 * D;
+    for (int64_t e = tid; e < n; e += kStatThreads) {
+        const float v = part[e];
+        if ((e / D) & 1) z = fmaxf(z, v); else a = fminf(a, v);   // [pair][min row | max row][D]
+    }
+    a = wave_min(a);
+    z = wave_max(z);
+    if ((tid & 63) == 0) { smn[tid >> 6] = a; smx[tid >> 6] = z; }
+    __syncthreads();
+    if (tid == 0) {
+        for (int w = 0; w < kStatThreads / kWave; ++w) { a = fminf(a, smn[w]); z = fmaxf(z, smx[w]); }
+        const float x_min = rnd<DT>(a * clip);
+        const float x_max = rnd<DT>(z * clip);
+        const float diff = rnd<DT>(x_max - x_min);
+        const float s = rnd<DT>(diff * __fdiv_rn(1.0f, levels));
+        st[0] = s;
+        st[1] = rnd<DT>(__fdiv_rn(-x_min, s));
+    }
+    __syncthreads();
+    const float s = st[0], zp = st[1];
+    const bool monotone = s > 0.0f && s < INFINITY && zp == zp;
+    const int nlev = static_cast<int>(levels);
+    if (tid < 3) {
+        const int k = tid + 1;
+        float t = NAN;
+        if (monotone && k <= nlev) {
+            int lo = Keys<DT>::lo, hi = Keys<DT>::hi;
+            if (quant_value<DT>(key_value<DT>(hi), s, zp, levels) >= static_cast<float>(k)) {
+                if (quant_value<DT>(key_value<DT>(lo), s, zp, levels) >= static_cast<float>(k)) {
+                    hi = lo;
+                } else {
+                    while (hi - lo > 1) {
+                        const int mid = lo + (hi - lo) / 2;
+                        if (quant_value<DT>(key_value<DT>(mid), s, zp, levels) >= static_cast<float>(k)) hi = mid;
+                        else lo = mid;
+                    }
+                }
+                t = key_value<DT>(hi);
+            }
+        }
+        if (!monotone) t = (k == 2) ? 1.0f : NAN;   // same marker as stats_kernel: emit evaluates the chain itself
+        st[2 + tid] = t;
+    }
+    __syncthreads();
+    for (int d = tid; d < D; d += kStatThreads) {
+        scale_row[d] = static_cast<uint16_t>(Cvt<DT>::from_float(s));
+        zero_row[d] = static_cast<uint16_t>(Cvt<DT>::from_float(zp));
+        thr_row[d] = st[2];
+        thr_row[D + d] = st[3];
+        thr_row[2 * D + d] = st[4];
+    }
+    if (tid == 0) {
+        scale1[0] = static_cast<uint16_t>(Cvt<DT>::from_float(s));
+        zero1[0] = static_cast<uint16_t>(Cvt<DT>::from_float(zp));
+    }
+}
+
 // ---- 3. emit -----------------------------------------------------------------
 // XQ = false: packed codes (B, H, T, D*BITS/8).  XQ = true: the unpacked code
 // values as storage-dtype numbers in a contiguous (B, T, H, D) tensor.
@@ -208,12 +282,13 @@ __global__ __launch_bounds__(kQThreads) void emit_kernel(const uint16_t* __restr
     const int t1 = min(g.T, t0 + g.chunk);
     const uint16_t* base = x + b * g.sb + h * g.sh + lane * 8;
     const int64_t bh = static_cast<int64_t>(b) * g.H + h;
+    const int64_t sbh = g.shared_stats ? 0 : bh;   // row of the statistics / threshold arrays
     constexpr float levels = static_cast<float>((1 << BITS) - 1);
 
     float s[8], zp[8];
     {
-        uint4 sv = *reinterpret_cast<const uint4*>(scale + bh * g.D + lane * 8);
-        uint4 zv = *reinterpret_cast<const uint4*>(zero + bh * g.D + lane * 8);
+        uint4 sv = *reinterpret_cast<const uint4*>(scale + sbh * g.D + lane * 8);
+        uint4 zv = *reinterpret_cast<const uint4*>(zero + sbh * g.D + lane * 8);
         unpack8<DT>(sv, s);
         unpack8<DT>(zv, zp);
     }
@@ -222,7 +297,7 @@ __global__ __launch_bounds__(kQThreads) void emit_kernel(const uint16_t* __restr
     float th[3][8];
     bool slow = false;
     {
-        const float4* tp = reinterpret_cast<const float4*>(thr + bh * 3 * g.D + lane * 8);
+        const float4* tp = reinterpret_cast<const float4*>(thr + sbh * 3 * g.D + lane * 8);
 #pragma unroll
         for (int k = 0; k < 3; ++k) {
             const float4 a = tp[k * (g.D >> 2)], c4 = tp[k * (g.D >> 2) + 1];
@@ -595,6 +670,32 @@ static int run_quant(const void* x, QuantGeom g, int bits, float clip, uint8_t* 
     return CQ_OK;
 }
 
+// quant(per_channel=False): partial min / max, whole-tensor statistics, emit of the unpacked codes.
+template <typename DT>
+static int run_quant_tensor(const void* x, QuantGeom g, int bits, float clip, void* xq, void* scale1, void* zero1,
+                            float* ws, hipStream_t st) {
+    dim3 grid(g.nchunk, g.H, g.B);
+    const uint16_t* xp = static_cast<const uint16_t*>(x);
+    hipLaunchKernelGGL(minmax_partial_kernel<DT>, grid, dim3(kQThreads), 0, st, xp, g, ws);
+    CQ_LAUNCH_CHECK();
+    const float levels = static_cast<float>((1 << bits) - 1);
+    const int64_t npairs = static_cast<int64_t>(g.B) * g.H * g.nchunk;
+    float* thr = ws + static_cast<size_t>(npairs) * 2 * g.D;            // 3 * D thresholds
+    uint16_t* srow = reinterpret_cast<uint16_t*>(thr + 3 * g.D);         // D scales, then D zero-points
+    uint16_t* zrow = srow + g.D;
+    hipLaunchKernelGGL(tensor_stats_kernel<DT>, dim3(1), dim3(kStatThreads), 0, st, ws, npairs, g.D, clip, levels, srow,
+                       zrow, thr, static_cast<uint16_t*>(scale1), static_cast<uint16_t*>(zero1));
+    CQ_LAUNCH_CHECK();
+    g.shared_stats = 1;
+    uint16_t* xqp = static_cast<uint16_t*>(xq);
+    if (bits == 1)
+        hipLaunchKernelGGL((emit_kernel<DT, 1, true>), grid, dim3(kQThreads), 0, st, xp, g, srow, zrow, thr, nullptr, xqp);
+    else
+        hipLaunchKernelGGL((emit_kernel<DT, 2, true>), grid, dim3(kQThreads), 0, st, xp, g, srow, zrow, thr, nullptr, xqp);
+    CQ_LAUNCH_CHECK();
+    return CQ_OK;
+}
+
 static int quant_entry(const void* x, int dtype, int B, int T, int H, int D, int64_t sb, int64_t st, int64_t sh,
                        int bits, float clip, uint8_t* codes, void* xq, void* scale, void* zero, void* ws,
                        size_t ws_bytes, cq_stream_t stream) {
@@ -760,8 +861,9 @@ extern "C" {
 
 size_t cq_quantize_pack_workspace(int B, int T, int H, int D) {
     if (B < 1 || T < 1 || H < 1 || D < 1) return 0;
-    // partial min / max per chunk, then three thresholds per channel
-    return static_cast<size_t>(B) * H * (static_cast<size_t>(cq::pick_chunks(B, T, H)) * 2 + 3) * D * sizeof(float);
+    // partial min / max per chunk, then three thresholds per channel (+ one row of statistics in the
+    // storage dtype for the whole-tensor mode of cq_quant_tensor)
+    return (static_cast<size_t>(B) * H * (static_cast<size_t>(cq::pick_chunks(B, T, H)) * 2 + 3) + 4) * D * sizeof(float);
 }
 
 int cq_quantize_pack(const void* x, int dtype, int B, int T, int H, int D, int64_t stride_b, int64_t stride_t,
@@ -814,6 +916,32 @@ int cq_quant(const void* x, int dtype, int B, int T, int H, int D, int64_t strid
     if (!x_q) return CQ_ERR_NULL;
     return cq::quant_entry(x, dtype, B, T, H, D, stride_b, stride_t, stride_h, bits, clip, nullptr, x_q, scale,
                            zero, workspace, workspace_bytes, stream);
+}
+
+int cq_quant_tensor(const void* x, int dtype, int B, int T, int H, int D, int64_t stride_b, int64_t stride_t,
+                    int64_t stride_h, int bits, float clip, void* x_q, void* scale1, void* zero1, void* workspace,
+                    size_t workspace_bytes, cq_stream_t stream) {
+    if (!x || !x_q || !scale1 || !zero1) return CQ_ERR_NULL;
+    if (dtype != CQ_BF16 && dtype != CQ_FP16) return CQ_ERR_DTYPE;
+    if (bits != 1 && bits != 2) return CQ_ERR_UNSUPPORTED;
+    if (B < 1 || T < 1 || H < 1 || (D != 64 && D != 128 && D != 256)) return CQ_ERR_SHAPE;
+    if (H > 65535 || B > 65535) return CQ_ERR_SHAPE;
+    if ((stride_b % 8) || (stride_t % 8) || (stride_h % 8) || !cq::aligned16(x) || !cq::aligned16(x_q) ||
+        (reinterpret_cast<uintptr_t>(scale1) & 1u) || (reinterpret_cast<uintptr_t>(zero1) & 1u))
+        return CQ_ERR_ALIGN;
+    const size_t need = cq_quantize_pack_workspace(B, T, H, D);
+    if (!workspace || workspace_bytes < need || !cq::aligned16(workspace)) return CQ_ERR_WORKSPACE;
+    cq::QuantGeom g = {};
+    g.B = B; g.T = T; g.H = H; g.D = D;
+    g.sb = stride_b; g.st = stride_t; g.sh = stride_h;
+    g.nchunk = cq::pick_chunks(B, T, H);
+    g.chunk = (T + g.nchunk - 1) / g.nchunk;
+    g.dT.set(static_cast<uint32_t>(T));
+    g.dH.set(static_cast<uint32_t>(H));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == CQ_BF16)
+        return cq::run_quant_tensor<cq::BF16>(x, g, bits, clip, x_q, scale1, zero1, static_cast<float*>(workspace), s);
+    return cq::run_quant_tensor<cq::FP16>(x, g, bits, clip, x_q, scale1, zero1, static_cast<float*>(workspace), s);
 }
 
 int cq_encode(const void* idx, int idx_dtype, int64_t rows, int D, int bits, uint8_t* out, cq_stream_t stream) {

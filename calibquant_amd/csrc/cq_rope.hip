@@ -4,8 +4,11 @@
 //
 // The reference does this with a chain of torch ops per layer and token
 // (patch_internvl.py:219-234 split, :258-260 and :119-138 rotary embedding,
-// :264-266 torch.cat append).  Arithmetic follows that chain op for op, rounding to
-// the storage dtype after every multiply and add, so results are bit-identical to it.
+// :264-266 torch.cat append).  Arithmetic follows the chain that runs there op for op:
+// `copy_().mul_(cos)` rounds x * cos to the storage dtype, then `addcmul_(rotate_half(x), sin)`
+// adds the product rotate_half(x) * sin in fp32 and rounds once (patch_internvl.py:125-128):
+// rnd(rnd(x * cos) + rot * sin).  The product of two 16-bit values is exact in fp32, so a
+// fused or an unfused multiply-add give the same bits.
 #include "cq_common.h"
 
 #pragma clang fp contract(off)
@@ -52,9 +55,9 @@ __global__ void rope_append_kernel(RopeGeom g) {
     const uint16_t* c = g.cos + p * kRD;
     const uint16_t* sn = g.sin + p * kRD;
     const float x1 = Cvt<DT>::to_float(lo), x2 = Cvt<DT>::to_float(hi);
-    // x * cos + rotate_half(x) * sin with rotate_half(x) = (-x2, x1)
-    const float o1 = rnd<DT>(rnd<DT>(x1 * Cvt<DT>::to_float(c[d])) + rnd<DT>(-x2 * Cvt<DT>::to_float(sn[d])));
-    const float o2 = rnd<DT>(rnd<DT>(x2 * Cvt<DT>::to_float(c[d + 64])) + rnd<DT>(x1 * Cvt<DT>::to_float(sn[d + 64])));
+    // rnd(rnd(x * cos) + rotate_half(x) * sin) with rotate_half(x) = (-x2, x1); the second product stays fp32
+    const float o1 = rnd<DT>(rnd<DT>(x1 * Cvt<DT>::to_float(c[d])) + (-x2 * Cvt<DT>::to_float(sn[d])));
+    const float o2 = rnd<DT>(rnd<DT>(x2 * Cvt<DT>::to_float(c[d + 64])) + (x1 * Cvt<DT>::to_float(sn[d + 64])));
     uint16_t* o;
     if (s < g.G) {
         o = g.q_out + ((static_cast<int64_t>(b) * g.Hkv + hkv) * g.G + s) * kRD;

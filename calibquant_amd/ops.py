@@ -104,6 +104,33 @@ def quant_codes(x: torch.Tensor, bits: int, clip: float):
     return xq, scale, zero
 
 
+def quant_codes_tensor(x: torch.Tensor, bits: int, clip: float):
+    """The unfused quantiser with one minimum / maximum over the whole tensor (the reference's
+    `per_channel=False`): x (..., D) -> (x_q shaped like x holding the integer codes, scale (), zero ())."""
+    _need_gpu(x, "x")
+    dt = _storage_dtype(x, "x")
+    shape = x.shape
+    if x.dim() == 4 and x.stride(3) == 1:
+        x4 = x
+    else:
+        if x.dim() < 1 or shape[-1] not in (64, 128, 256):
+            raise _lib.CalibQuantError("x must end in an axis of 64, 128 or 256 elements")
+        x4 = x.reshape(1, -1, 1, shape[-1])
+        if x4.stride(3) != 1:
+            x4 = x4.contiguous()
+    B, T, H, D = x4.shape
+    lib = _lib.load()
+    xq = torch.empty((B, T, H, D), dtype=x.dtype, device=x.device)
+    stats = torch.empty(16, dtype=x.dtype, device=x.device)        # scale at [0], zero-point at [8]
+    ws = _workspace(lib.cq_quantize_pack_workspace(B, T, H, D), x.device)
+    with torch.cuda.device(x.device):
+        rc = lib.cq_quant_tensor(x4.data_ptr(), dt, B, T, H, D, x4.stride(0), x4.stride(1), x4.stride(2),
+                                 bits, float(clip), xq.data_ptr(), stats[0:].data_ptr(), stats[8:].data_ptr(),
+                                 ws.data_ptr(), ws.numel(), _stream(x))
+    _lib.check(rc, "cq_quant_tensor")
+    return xq.view(shape), stats[0], stats[8]
+
+
 def encode_indices(idx: torch.Tensor, bits: int) -> torch.Tensor:
     """Pack integer indices (..., D) into uint8 (..., D*bits/8), first index in the high bits."""
     _need_gpu(idx, "idx")
@@ -121,7 +148,10 @@ def encode_indices(idx: torch.Tensor, bits: int) -> torch.Tensor:
 
 def lut_vecmat(kind: str, lut: torch.Tensor, a: torch.Tensor, enc: torch.Tensor, bits: int) -> torch.Tensor:
     """kind 'qk': a (M, D), enc (M, T, D*bits/8) -> (M, T) fp16;
-    kind 'pv': a (M, T), enc (M, T, D*bits/8) -> (M, D) fp16."""
+    kind 'pv': a (M, T), enc (M, T, D*bits/8) -> (M, D) fp16.
+    `lut` may hold fewer than 2**bits entries: a code without an entry contributes 0."""
+    if lut.numel() < 1:
+        raise _lib.CalibQuantError("lut must hold at least one entry")
     for t, n in ((lut, "lut"), (a, "a"), (enc, "enc")):
         _need_gpu(t, n)
     lut, a, enc = lut.contiguous(), a.contiguous(), enc.contiguous()
@@ -130,7 +160,7 @@ def lut_vecmat(kind: str, lut: torch.Tensor, a: torch.Tensor, enc: torch.Tensor,
     out = torch.empty((M, T if kind == "qk" else D), dtype=torch.float16, device=a.device)
     fn = _lib.load().cq_lut_vecmat_qk if kind == "qk" else _lib.load().cq_lut_vecmat_pv
     with torch.cuda.device(a.device):
-        rc = fn(lut.data_ptr(), _DT[lut.dtype], a.data_ptr(), _DT[a.dtype], enc.data_ptr(), M, T, D, bits,
+        rc = fn(lut.data_ptr(), _DT[lut.dtype], lut.numel(), a.data_ptr(), _DT[a.dtype], enc.data_ptr(), M, T, D, bits,
                 out.data_ptr(), _stream(a))
     _lib.check(rc, f"cq_lut_vecmat_{kind}")
     return out

@@ -58,10 +58,15 @@ def rotate_half(x):
 
 
 def apply_rotary_pos_emb(q, k, cos, sin, position_ids, unsqueeze_dim=1):
-    """Rotary position embedding of q and k (patch_internvl.py:119-138)."""
+    """Rotary position embedding of q and k with the rounding of the ops the reference runs
+    (patch_internvl.py:125-128, 131-134): `x * cos` is rounded to the storage dtype, then
+    `addcmul` adds `rotate_half(x) * sin` in fp32 and rounds the sum once.  (The two-rounding
+    form `(x * cos) + (rotate_half(x) * sin)` is the commented-out line :123 and differs from
+    this by one unit in the last place in about a quarter of the elements.)  The inputs are
+    left untouched; the reference's `rotate_half` negates the upper half of its argument in place."""
     cos = cos[position_ids].unsqueeze(unsqueeze_dim)
     sin = sin[position_ids].unsqueeze(unsqueeze_dim)
-    return (q * cos) + (rotate_half(q) * sin), (k * cos) + (rotate_half(k) * sin)
+    return torch.addcmul(q * cos, rotate_half(q), sin), torch.addcmul(k * cos, rotate_half(k), sin)
 
 
 @torch.no_grad()
@@ -86,8 +91,8 @@ def custom_generate(self, pixel_values=None, input_ids=None, attention_mask=None
         input_embeds[selected] = vit_embeds.reshape(-1, C).to(input_embeds.device, input_embeds.dtype)
         image_token_num = int(vit_embeds.shape[0] * vit_embeds.shape[1] / B)
         os.environ["IMAGE_TOKEN_NUM"] = str(image_token_num)
-        for layer in lm.model.layers:
-            layer.attention.image_token_num = image_token_num
+        for layer in lm.model.layers:      # the explicit per-module channel; wins over the env var
+            layer.attention.cq_image_token_num = image_token_num
         input_embeds = input_embeds.reshape(B, N, C)
     else:
         input_embeds = lm.get_input_embeddings()(input_ids)
@@ -97,11 +102,15 @@ def custom_generate(self, pixel_values=None, input_ids=None, attention_mask=None
 
 
 def _image_token_num(self) -> int:
-    n = getattr(self, "image_token_num", None)
+    """The image token count of this forward: the explicit override `cq_image_token_num` on the
+    module if a caller set one (`custom_generate` does), else the `IMAGE_TOKEN_NUM` environment
+    variable, re-read on every forward as the reference does (patch_internvl.py:189,251) - a caller
+    that only updates the variable between prompts gets the new count."""
+    n = getattr(self, "cq_image_token_num", None)
     if n is None:
         env = os.environ.get("IMAGE_TOKEN_NUM")
         if env is None:
-            raise CalibQuantError("image token count unknown: set attention.image_token_num or IMAGE_TOKEN_NUM")
+            raise CalibQuantError("image token count unknown: set attention.cq_image_token_num or IMAGE_TOKEN_NUM")
         n = int(env)
     return int(n)
 
@@ -196,12 +205,18 @@ def forward_internlm2_calibquant(self, hidden_states: torch.Tensor, attention_ma
         else:
             past_key_value = None
         # full-precision causal attention over the whole prompt, in query chunks
+        # The reference hands `attention_mask` to `_flash_attention_forward` as it is
+        # (patch_internvl.py:465-467), which takes a (B, kv) key-padding mask.  Any other layout
+        # (the 4-D additive masks of the eager / SDPA attention classes) cannot be honoured by that
+        # call: refuse it instead of attending to the padding.
+        if attention_mask is not None and attention_mask.dim() != 2:
+            raise CalibQuantError(f"prefill: attention_mask must be a (B, kv) key-padding mask or None, got a "
+                                  f"{attention_mask.dim()}-D tensor of shape {tuple(attention_mask.shape)}")
         q_t, k_t, v_t = query_states.transpose(1, 2), key_states.transpose(1, 2), value_states.transpose(1, 2)
         outs = []
         for i in range(0, q_len, CHUNK_SIZE):
             outs.append(self._flash_attention_forward(q_t[:, i:i + CHUNK_SIZE], k_t[:, :i + CHUNK_SIZE],
-                                                      v_t[:, :i + CHUNK_SIZE], attention_mask if attention_mask is None
-                                                      or attention_mask.dim() == 2 else None,
+                                                      v_t[:, :i + CHUNK_SIZE], attention_mask,
                                                       q_t[:, :i + CHUNK_SIZE].shape[1]))
         attn_output = torch.cat(outs, dim=1).reshape(bsz, q_len, self.hidden_size)
         return self.wo(attn_output), None, past_key_value
@@ -250,7 +265,7 @@ def _attend(self, q1, k_res, v_res, mask):
 def _decode_step_fused(self, qkv, position_ids, past_key_value, attention_mask, use_cache):
     """One decode step with the split of the fused projection, the rotary embedding of q and k and
     the append of the new key / value row in one launch (`cq_rope_append`, bit-identical to the
-    chain of torch ops of patch_internvl.py:119-138, 219-266), then the fused attention launch."""
+    torch ops that run at patch_internvl.py:125-134, 219-266), then the fused attention launch."""
     bsz = qkv.shape[0]
     G, D, Hq = self.num_key_value_groups, self.head_dim, self.num_heads
     Hkv = Hq // G

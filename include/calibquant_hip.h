@@ -92,6 +92,19 @@ int cq_quant(const void* x, int dtype, int B, int T, int H, int D,
              void* x_q, void* scale, void* zero,
              void* workspace, size_t workspace_bytes, cq_stream_t stream);
 
+/* quant() with per_channel=False (calibquant.py:29-31): one minimum and one
+ * maximum over the whole tensor (`x.min() * scale`, `x.max() * scale`), then
+ * the same op chain as above.  x and x_q as for cq_quant; scale1 and zero1
+ * receive a single storage-dtype element each (the reference returns 0-d
+ * tensors).  Not called by the attention path (patch_internvl.py:181,187 pass
+ * per_channel=True); provided so that the operator's whole signature works.
+ * workspace: cq_quantize_pack_workspace(B, T, H, D) bytes. */
+int cq_quant_tensor(const void* x, int dtype, int B, int T, int H, int D,
+                    int64_t stride_b, int64_t stride_t, int64_t stride_h,
+                    int bits, float clip,
+                    void* x_q, void* scale1, void* zero1,
+                    void* workspace, size_t workspace_bytes, cq_stream_t stream);
+
 /* encode(): pack `rows` rows of D integer indices, 8/bits per byte,
  * first index in the most significant bits (calibquant.py:114-137).
  * idx_dtype: CQ_I64, CQ_I32, CQ_U8, or CQ_BF16/CQ_FP16 numbers holding
@@ -101,16 +114,19 @@ int cq_encode(const void* idx, int idx_dtype, int64_t rows, int D, int bits,
 
 /* fused_kernel(): c[m, t] = sum_d a[m, d] * lut[code[m, t, d]], fp32
  * accumulation, fp16 output (calibquant.py:54-111).  a: (M, D) in a_dtype
- * (CQ_BF16/CQ_FP16/CQ_FP32); enc: (M, T, D*bits/8); lut: 2^bits entries in
- * lut_dtype; out: (M, T) fp16. */
-int cq_lut_vecmat_qk(const void* lut, int lut_dtype, const void* a, int a_dtype,
+ * (CQ_BF16/CQ_FP16/CQ_FP32); enc: (M, T, D*bits/8); lut: lut_len entries in
+ * lut_dtype (the reference's table holds the levels found in the first
+ * 10 000 codes, patch_internvl.py:318-329, so it may be shorter than 2^bits:
+ * a code without an entry contributes 0 and nothing past the table is read);
+ * out: (M, T) fp16.  M < 2^31, T <= 65 535 * 256. */
+int cq_lut_vecmat_qk(const void* lut, int lut_dtype, int lut_len, const void* a, int a_dtype,
                      const uint8_t* enc, int64_t M, int T, int D, int bits,
                      void* out_fp16, cq_stream_t stream);
 
 /* fused_kernel_wv(): c[m, d] = sum_t a[m, t] * lut[code[m, t, d]], fp32
  * accumulation, fp16 output (calibquant.py:192-276).  a: (M, T);
  * enc: (M, T, D*bits/8); out: (M, D) fp16. */
-int cq_lut_vecmat_pv(const void* lut, int lut_dtype, const void* a, int a_dtype,
+int cq_lut_vecmat_pv(const void* lut, int lut_dtype, int lut_len, const void* a, int a_dtype,
                      const uint8_t* enc, int64_t M, int T, int D, int bits,
                      void* out_fp16, cq_stream_t stream);
 
@@ -185,7 +201,9 @@ size_t cq_decode_attn_workspace(const cq_decode_args* args);
 int cq_decode_attn(const cq_decode_args* args, cq_stream_t stream);
 
 /* What cq_decode_attn would launch for these arguments (pointers are not
- * looked at; host-only, no device call).  No counterpart in the reference,
+ * looked at; nothing is launched - the only device call is a query of the
+ * current device's compute-unit count, made once per process; a whole MI355X,
+ * 256 units, is assumed when there is no device).  No counterpart in the reference,
  * whose Triton kernels re-autotune per shape (calibquant.py:54-76,192-218):
  * here the choice is a pure function of the shape, and a caller can read it. */
 typedef struct cq_decode_plan {
@@ -203,16 +221,21 @@ int cq_decode_attn_plan(const cq_decode_args* args, cq_decode_plan* plan);
 /* ------------------------------------------------------------------------
  * Decode-step glue, one launch per layer and token: the (h gs d) split of
  * the fused wqkv output (patch_internvl.py:219-234), rotary embedding of the
- * query and key heads (patch_internvl.py:119-138, 258-260; x*cos +
- * rotate_half(x)*sin, rounded to the storage dtype after every op as the
- * chain of torch ops does) and the append of the new key / value row to the
+ * query and key heads (patch_internvl.py:119-138, 258-260) with the rounding
+ * of the ops that run there: x*cos rounded to the storage dtype
+ * (`copy_().mul_()`, :125), then rotate_half(x)*sin added in fp32 and the sum
+ * rounded once (`addcmul_`, :127) - not the two-rounding form of the
+ * commented-out line :123 - and the append of the new key / value row to the
  * full-precision window (the reference's torch.cat, patch_internvl.py:264-266).
  * qkv: (B, Hkv, Hq/Hkv + 2, D) contiguous, one token per sample; cos_table,
  * sin_table: (table_rows, D) in the storage dtype; pos: device int64,
- * sample b at pos[b*pos_stride] (clamped to the table); q_out: (B, Hq, D)
+ * sample b at pos[b*pos_stride] (a position outside [0, table_rows) is
+ * clamped to the nearest table row without an error: the caller sizes the
+ * tables to cover the positions it passes); q_out: (B, Hq, D)
  * contiguous; k_win, v_win: (B, Hkv, capacity, D) through element strides;
  * row_dev: device int64, the window row that receives the new key / value
- * (nothing is written if it is outside [0, capacity)).  Position and row are
+ * (if it is outside [0, capacity) the key / value row is dropped without an
+ * error: the caller keeps the row inside the window).  Position and row are
  * read on the device, so a recorded launch can be replayed. */
 int cq_rope_append(const void* qkv, int dtype, int B, int Hq, int Hkv, int D,
                    const void* cos_table, const void* sin_table, int64_t table_rows,

@@ -29,9 +29,15 @@ Pinning status (what each function is checked against in tests/):
   decode_attention_refchain   informational mixed-precision chain; its
                         rounding sequence follows the reference text but
                         no reference-held vector exists for it: parity unpinned
-  kivi_quantize_pack / kivi_pv   closed form + little-endian word packing
-                        (numpy.packbits bitorder='little' at b=1), group
-                        min / range, midpoint rule                       pinned
+  quant(per_channel=False)   torch CPU eager chain with x.min() / x.max()  pinned
+  rope                  torch CPU running the reference's op sequence
+                        (copy_().mul_(), in-place rotate_half, addcmul_);
+                        differs from the two-rounding form in ~25 % of
+                        the elements, which the test also checks        pinned
+  kivi_quantize_pack / kivi_pv   torch CPU eager chain of new_pack.py:64-72
+                        (levels_division="true"), closed form + little-endian
+                        word packing (numpy.packbits bitorder='little' at
+                        b=1), group min / range, midpoint rule           pinned
   decode_attention(v_token_group)   python-loop brute force on explicitly
                         dequantised scale*code + minimum values          pinned
 """
@@ -80,7 +86,7 @@ def _f32(x):
 # a1: quant  (calibquant.py:24-42)
 # --------------------------------------------------------------------------
 def quant(x, bits: int, clip: float = 1.0, dtype: str = "bf16",
-          levels_division: str = "reciprocal"):
+          levels_division: str = "reciprocal", per_channel: bool = True):
     """Per-channel b-bit min-max quantiser, `post_scale=True` branch.
 
     x: (B, T, H, D) storage-dtype values (float32 container).  The reduction
@@ -100,13 +106,21 @@ def quant(x, bits: int, clip: float = 1.0, dtype: str = "bf16",
     levels_division: torch's GPU kernel for `tensor / python_scalar` multiplies
     by the fp32 reciprocal of the scalar ("reciprocal", the behaviour on the
     device the reference hard-wires at calibquant.py:11); torch's CPU kernel
-    divides ("true").  They coincide for 1-bit (levels == 1)."""
+    divides ("true").  They coincide for 1-bit (levels == 1).
+
+    per_channel=False: one minimum and one maximum over the whole tensor
+    (`x.min() * scale`, `x.max() * scale`, calibquant.py:29-31); scale and
+    zero are then 0-d arrays."""
     x = _f32(x)
     levels = float(2 ** bits - 1)
     c = np.float32(clip)
     with np.errstate(all="ignore"):
-        x_min = round_to(x.min(axis=1, keepdims=True) * c, dtype)
-        x_max = round_to(x.max(axis=1, keepdims=True) * c, dtype)
+        if per_channel:
+            x_min = round_to(x.min(axis=1, keepdims=True) * c, dtype)
+            x_max = round_to(x.max(axis=1, keepdims=True) * c, dtype)
+        else:
+            x_min = round_to(x.min() * c, dtype)
+            x_max = round_to(x.max() * c, dtype)
         # numpy min/max propagate NaN like torch.amin/amax
         diff = round_to(x_max - x_min, dtype)
         if levels_division == "reciprocal":
@@ -371,7 +385,8 @@ def decode_attention_refchain(q, codes_k, codes_v, k_scale, k_zero, v_scale,
 # a12: KIVI-style per-token value quantiser  (qjl/new_pack.py:53-82) and its
 # consumer (qjl/csrc/quantization.cu:67-132)
 # --------------------------------------------------------------------------
-def kivi_quantize_pack(v, group_size: int, bits: int, dtype: str = "bf16"):
+def kivi_quantize_pack(v, group_size: int, bits: int, dtype: str = "bf16",
+                       levels_division: str = "reciprocal"):
     """Per-token, per-group-of-channels min-max quantiser with 32/bits codes
     per int32 word, first code in the LEAST significant bits.
 
@@ -389,7 +404,10 @@ def kivi_quantize_pack(v, group_size: int, bits: int, dtype: str = "bf16"):
     with np.errstate(all="ignore"):
         mn = g.min(-1)
         mx = g.max(-1)
-        scale = round_to(round_to(mx - mn, dtype) * (np.float32(1.0) / np.float32(L)), dtype)
+        if levels_division == "reciprocal":   # torch's device kernel for tensor / python scalar
+            scale = round_to(round_to(mx - mn, dtype) * (np.float32(1.0) / np.float32(L)), dtype)
+        else:                                  # torch's CPU kernel divides
+            scale = round_to(round_to(mx - mn, dtype) / np.float32(L), dtype)
         y = round_to(g - mn[..., None], dtype)
         y = round_to(y / scale[..., None], dtype)
         y = np.where(np.isnan(y), y, np.clip(y, 0, L))
@@ -419,6 +437,29 @@ def kivi_pv(p, words, scale, mn, group_size: int, bits: int) -> np.ndarray:
     s = np.repeat(_f32(scale), group_size, axis=-1)
     m = np.repeat(_f32(mn), group_size, axis=-1)
     return np.einsum("bht,bhtd->bhd", _f32(p), s * code + m, dtype=np.float32)
+
+
+# --------------------------------------------------------------------------
+# rotary position embedding  (patch_internvl.py:110-138)
+# --------------------------------------------------------------------------
+def rope(x, cos, sin, dtype: str = "bf16") -> np.ndarray:
+    """Rotary embedding with the rounding of the ops that run in the reference.
+
+    x: (..., D) storage-dtype values; cos, sin broadcastable to x (already
+    gathered by position id).  The reference computes (patch_internvl.py:125-128)
+        e = empty_like(x); e.copy_(x).mul_(cos)      -> rnd(x * cos)
+        tmp = rotate_half(x)                         -> (-x2, x1), exact
+        e.addcmul_(tmp, sin)                         -> rnd(e + tmp * sin)
+    where addcmul works in fp32 and rounds once: the product tmp * sin of two
+    16-bit values is exact in fp32, the fp32 sum is rounded to fp32 and then
+    to the storage dtype.  (The commented-out line :123 would round the second
+    product to the storage dtype as well.)"""
+    x = _f32(x)
+    cos, sin = _f32(cos), _f32(sin)
+    h = x.shape[-1] // 2
+    rot = np.concatenate([-x[..., h:], x[..., :h]], axis=-1)
+    first = round_to(x * cos, dtype)
+    return round_to((first + rot * sin).astype(np.float32), dtype)
 
 
 # --------------------------------------------------------------------------

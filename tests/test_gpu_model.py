@@ -28,7 +28,7 @@ def test_patched_forward_decode_matches_oracle_on_one_layer():
     torch.manual_seed(1)
     cfg = InternLM2Config.tiny()
     att = InternLM2Attention(cfg).cuda().to(torch.bfloat16)
-    att.cq_sprompt_len, att.image_token_num = 5, 200
+    att.cq_sprompt_len, att.cq_image_token_num = 5, 200
     B, S, T, TXT = 2, 5, 200, 11
     N = S + T + TXT
     x = torch.randn(B, N, cfg.hidden_size, device="cuda", dtype=torch.bfloat16)
@@ -78,7 +78,7 @@ def test_fused_decode_step_equals_the_unfused_op_chain(dtype):
     for fused in (True, False):
         torch.manual_seed(7)
         att = InternLM2Attention(cfg).cuda().to(dtype)
-        att.cq_sprompt_len, att.image_token_num = S, T
+        att.cq_sprompt_len, att.cq_image_token_num = S, T
         x = torch.randn(B, N, cfg.hidden_size, device="cuda", dtype=dtype)
         pos = torch.arange(N, device="cuda")[None].expand(B, N)
         with torch.no_grad():
@@ -123,7 +123,7 @@ def test_patched_model_without_image_tokens_equals_the_fp_model():
             b0, b1 = two_steps()
             pi.patch_model(m, "calibquant", sprompt_len=0)
             for layer in lm.model.layers:
-                layer.attention.image_token_num = 0
+                layer.attention.cq_image_token_num = 0
             p0, p1 = two_steps()
         assert torch.allclose(b0, p0, atol=3e-2, rtol=3e-2)
         assert torch.allclose(b1, p1, atol=3e-2, rtol=3e-2)
@@ -191,7 +191,7 @@ def test_static_decoder_graph_replays_equal_eager_steps(quantized, fp_kernel):
             if quantized:
                 pi.patch_model(m, "calibquant")
                 for layer in lm.model.layers:
-                    layer.attention.image_token_num = T
+                    layer.attention.cq_image_token_num = T
             runs = []
             for use_graph in (False, True):
                 logits, past = _prefill(m, ids, pix)
@@ -229,7 +229,7 @@ def test_patched_model_with_per_token_values():
     torch.manual_seed(9)
     cfg = InternLM2Config.tiny()
     att = InternLM2Attention(cfg).cuda().to(torch.bfloat16)
-    att.cq_sprompt_len, att.image_token_num, att.cq_v_mode = 4, 300, "token"
+    att.cq_sprompt_len, att.cq_image_token_num, att.cq_v_mode = 4, 300, "token"
     B, S, T, TXT = 2, 4, 300, 6
     N = S + T + TXT
     x = torch.randn(B, N, cfg.hidden_size, device="cuda", dtype=torch.bfloat16)
@@ -253,3 +253,31 @@ def test_patched_model_with_per_token_values():
         ref = att.wo(torch.from_numpy(want).cuda().to(torch.bfloat16).reshape(B, 1, -1))
         err = (out_d.float() - ref.float()).abs()
         assert err.max().item() < 2e-2 and err.mean().item() < 2e-3
+
+
+def test_two_prefills_follow_the_environment_variable(monkeypatch):
+    """Two prompts through the patched forward with only IMAGE_TOKEN_NUM updated in between
+    (no custom_generate, no attribute): each prefill quantises its own image slice, and a 4-D
+    prefill mask is refused instead of being dropped."""
+    from calibquant_amd import patch_internvl as pi
+    from calibquant_amd._lib import CalibQuantError
+    from calibquant_amd.internlm2 import InternLM2Attention, InternLM2Config
+    torch.manual_seed(3)
+    cfg = InternLM2Config.tiny()
+    att = InternLM2Attention(cfg).cuda().to(torch.bfloat16)
+    att.cq_sprompt_len = 3
+    B = 2
+    with torch.no_grad():
+        for T in (200, 72):
+            monkeypatch.setenv("IMAGE_TOKEN_NUM", str(T))
+            N = 3 + T + 5
+            x = torch.randn(B, N, cfg.hidden_size, device="cuda", dtype=torch.bfloat16)
+            pos = torch.arange(N, device="cuda")[None].expand(B, N)
+            _, _, past = pi.forward_internlm2_calibquant(att, x, None, pos, None, False, True)
+            assert att.image_token_num == T and att.encoded_features_k.shape[2] == T
+            assert past[0].shape[2] == N - T
+            q, k, v = att.split_qkv(x)
+            cv, _, _ = O.quantize_pack(to_np(v[:, 3:3 + T]), 1, 0.3, "bf16")
+            assert np.array_equal(att.encoded_features_v.cpu().numpy(), cv)
+        with pytest.raises(CalibQuantError):
+            pi.forward_internlm2_calibquant(att, x, torch.zeros(B, 1, N, N, device="cuda"), pos, None, False, True)

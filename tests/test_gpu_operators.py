@@ -8,7 +8,7 @@ import pytest
 import torch
 
 from oracle import cq_oracle as O
-from tests.util import CLIPS, make_case, case_to_gpu, same_bits, to_gpu, to_np
+from tests.util import CLIPS, make_case, case_to_gpu, reference_rope_sequence, same_bits, to_gpu, to_np
 
 pytestmark = pytest.mark.gpu
 
@@ -53,6 +53,55 @@ def test_fused_kernels_honour_an_arbitrary_table(cq, bits):
     # fp32 accumulation order differs from numpy's: allow one fp16 ulp
     assert np.allclose(to_np(qk), want_qk, rtol=2e-3, atol=2e-3)
     assert np.allclose(to_np(pv), want_pv, rtol=2e-3, atol=1e-4)
+
+
+@pytest.mark.parametrize("bits", [1, 2])
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+def test_quant_whole_tensor_mode(cq, bits, dtype):
+    """quant(per_channel=False) (calibquant.py:29-31): one min / max over the whole tensor; bit-exact
+    against the oracle and against torch-ROCm running the reference's op chain on the device."""
+    k, _ = O.synth_kv(3, 700, 4, 128, dtype, seed=4)
+    x = to_gpu(k, dtype)[:, :, 1:, :]                      # a strided view: heads 1..3
+    clip = CLIPS[bits][0]
+    x_q, s, z = cq.quant(x, bits=bits, per_channel=False, scale=clip, post_scale=True)
+    assert x_q.shape == x.shape and s.dim() == 0 and z.dim() == 0
+    oxq, os_, oz = O.quant(k[:, :, 1:, :], bits, clip, dtype, per_channel=False)
+    assert float(s) == float(os_) and float(z) == float(oz)
+    assert same_bits(to_np(x_q), oxq)
+    L = 2 ** bits - 1
+    mn, mx = x.min() * clip, x.max() * clip
+    st = (mx - mn) / L
+    zt = -mn / st
+    xq_t = torch.round(torch.clamp(x / st + zt, 0, L))
+    assert torch.equal(s, st) and torch.equal(z, zt) and torch.equal(x_q, xq_t)
+    deq, _, _ = cq.quant(x, bits=bits, per_channel=False, scale=clip, post_scale=False)
+    assert torch.equal(deq, st * (xq_t - zt))
+    # any shape ending in the channel axis
+    flat = to_gpu(k, dtype).reshape(-1, 128)
+    fq, fs, fz = cq.quant(flat, bits=bits, per_channel=False, scale=clip, post_scale=True)
+    o2 = O.quant(k, bits, clip, dtype, per_channel=False)
+    assert fq.shape == flat.shape and same_bits(to_np(fq), o2[0].reshape(-1, 128)) and float(fs) == float(o2[1])
+
+
+def test_fused_kernels_with_a_table_shorter_than_the_code_range(cq):
+    """The reference builds its table from the levels seen in the first 10 000 codes
+    (patch_internvl.py:318-329), so it can hold fewer than 2^bits entries: a code without an
+    entry contributes 0 and nothing past the table is read."""
+    rng = np.random.default_rng(1)
+    B, H, T, D, bits = 1, 2, 100, 128, 2
+    idx = rng.integers(0, 4, size=(B, H, T, D))
+    enc = O.encode(idx, bits)
+    a = O.round_to(rng.standard_normal((B, H, 1, D)), "bf16")
+    p = O.round_to(rng.random((B, H, 1, T)) / T, "fp16")
+    enc_g = torch.from_numpy(enc).cuda()
+    for n in (1, 3):
+        short = np.array([0.5, -1.0, 2.0][:n], np.float32)
+        full = np.concatenate([short, np.zeros(4 - n, np.float32)])
+        # the table sits at the very end of its allocation's used part: entries past it would be foreign memory
+        qk = cq.fused_kernel(to_gpu(short, "bf16"), to_gpu(a, "bf16"), enc_g, bits, 4)
+        pv = cq.fused_kernel_wv(to_gpu(short, "fp16"), to_gpu(p, "fp16"), enc_g, bits, 4)
+        assert np.allclose(to_np(qk), O.lut_vecmat_qk(full, a, enc, bits), rtol=2e-3, atol=2e-3)
+        assert np.allclose(to_np(pv), O.lut_vecmat_pv(full, p, enc, bits), rtol=2e-3, atol=1e-4)
 
 
 def test_unfused_reference_sequence_agrees_with_the_fused_kernel(cq):
@@ -115,9 +164,18 @@ def test_rope_append_equals_the_torch_op_chain_bit_for_bit(dtype, heads):
     q = v5[..., :G, :].reshape(B, 1, Hq, D).transpose(1, 2)
     k = v5[..., -2, :].transpose(1, 2)
     v = v5[..., -1, :].transpose(1, 2)
-    qr, kr = pi.apply_rotary_pos_emb(q, k, cos, sin, pos)
+    # (1) torch-ROCm running the reference's own op sequence on the device, (2) the oracle, (3) the
+    # package's Python helper: all four agree bit for bit
+    c1, s1 = cos[pos].unsqueeze(1), sin[pos].unsqueeze(1)
+    qr, kr = reference_rope_sequence(q, c1, s1), reference_rope_sequence(k, c1, s1)
     assert torch.equal(q_out, qr[:, :, 0])
     assert torch.equal(kwin[:, :, 17], kr[:, :, 0]) and torch.equal(vwin[:, :, 17], v[:, :, 0])
+    name = "bf16" if dtype == torch.bfloat16 else "fp16"
+    assert np.array_equal(to_np(q_out), O.rope(to_np(q[:, :, 0]), to_np(c1[:, 0]), to_np(s1[:, 0]), name))
+    qh, kh = pi.apply_rotary_pos_emb(q, k, cos, sin, pos)
+    assert torch.equal(qh, qr) and torch.equal(kh, kr)
+    two = q * c1 + pi.rotate_half(q) * s1              # the two-rounding form is a different function
+    assert not torch.equal(two, qr)
     kwin[:, :, 17] = 0
     vwin[:, :, 17] = 0
     assert not kwin.any() and not vwin.any()          # nothing else was written
@@ -149,7 +207,8 @@ def test_rope_append_full_batch_and_replay_by_device_counters():
         call.run()
         v5 = qkv.view(B, 1, Hkv, 2 + G, D)
         q = v5[..., :G, :].reshape(B, 1, Hq, D).transpose(1, 2)
-        qr, kr = pi.apply_rotary_pos_emb(q, v5[..., -2, :].transpose(1, 2), cos, sin, pos)
+        c1, s1 = cos[pos].unsqueeze(1), sin[pos].unsqueeze(1)
+        qr, kr = reference_rope_sequence(q, c1, s1), reference_rope_sequence(v5[..., -2, :].transpose(1, 2), c1, s1)
         assert torch.equal(q_out, qr[:, :, 0]) and torch.equal(kwin[:, :, step], kr[:, :, 0])
         assert torch.equal(vwin[:, :, step], v5[:, 0, :, -1, :])
         pos.add_(1)

@@ -116,8 +116,8 @@ def test_c_abi_rejects_bad_arguments_without_touching_the_gpu():
     a.T, a.B = 32768, 8
     ws = lib.cq_decode_attn_workspace(ctypes.byref(a))
     assert ws > 0 and ws % 4 == 0                                         # chunked path needs partials
-    # 8 token chunks of partial min / max, then 3 thresholds per channel
-    assert lib.cq_quantize_pack_workspace(64, 3328, 8, 128) == 64 * 8 * (8 * 2 + 3) * 128 * 4
+    # 8 token chunks of partial min / max, then 3 thresholds per channel, + 4 rows for the whole-tensor mode
+    assert lib.cq_quantize_pack_workspace(64, 3328, 8, 128) == (64 * 8 * (8 * 2 + 3) + 4) * 128 * 4
     a.T, a.B, a.v_mode = 64, 1, 7
     assert lib.cq_decode_attn(ctypes.byref(a), None) == -7                # unknown value layout
     assert lib.cq_quantize_pack_token(None, 0, 1, 1, 1, 128, 0, 0, 0, 1, 32, None, None, None, None) == -1
@@ -196,3 +196,26 @@ def test_internlm2_wqkv_interleave_matches_the_reference_rearrange():
     qkv = rearrange(att.wqkv(x), "b q (h gs d) -> b q h gs d", gs=2 + att.num_key_value_groups, d=att.head_dim)
     assert torch.equal(q, rearrange(qkv[..., : att.num_key_value_groups, :], "b q h gs d -> b q (h gs) d"))
     assert torch.equal(k, qkv[..., -2, :]) and torch.equal(v, qkv[..., -1, :])
+
+
+def test_image_token_count_is_reread_from_the_environment_every_forward(monkeypatch):
+    """The reference reads IMAGE_TOKEN_NUM on every forward (patch_internvl.py:189,251): a caller that
+    only updates the variable between prompts must get the new count; an explicit override on the
+    module wins; the attribute a forward publishes never feeds back into the next one."""
+    from calibquant_amd import patch_internvl as pi
+    from calibquant_amd._lib import CalibQuantError
+
+    class Att:
+        pass
+
+    att = Att()
+    monkeypatch.delenv("IMAGE_TOKEN_NUM", raising=False)
+    with pytest.raises(CalibQuantError):
+        pi._image_token_num(att)
+    monkeypatch.setenv("IMAGE_TOKEN_NUM", "3328")
+    att.image_token_num = pi._image_token_num(att)        # what a forward publishes on the module
+    assert att.image_token_num == 3328
+    monkeypatch.setenv("IMAGE_TOKEN_NUM", "512")           # second prompt, no custom_generate in between
+    assert pi._image_token_num(att) == 512
+    att.cq_image_token_num = 256                            # the explicit channel (custom_generate sets it)
+    assert pi._image_token_num(att) == 256

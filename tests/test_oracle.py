@@ -7,6 +7,7 @@ import pytest
 import torch
 
 from oracle import cq_oracle as O
+from tests.util import reference_rope_sequence
 
 TDT = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}
 
@@ -57,6 +58,45 @@ def test_quant_matches_torch_eager_chain(dtype, bits, clip):
         assert np.array_equal(s, s_t)
         assert np.array_equal(z, z_t)
         assert np.array_equal(xq, xq_t)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("bits,clip", [(1, 0.5), (2, 1)])
+def test_quant_whole_tensor_matches_torch_eager_chain(dtype, bits, clip):
+    """per_channel=False (calibquant.py:29-31): x.min() / x.max() over the whole tensor."""
+    k, _ = O.synth_kv(2, 65, 3, 64, dtype, seed=12)
+    xq, s, z = O.quant(k, bits, clip, dtype, levels_division="true", per_channel=False)
+    xt = _t(k, dtype)
+    L = 2 ** bits - 1
+    mn, mx = xt.min() * clip, xt.max() * clip
+    st = (mx - mn) / L
+    zt = -mn / st
+    xq_t = torch.round(torch.clamp(xt / st + zt, 0, L))
+    assert s.shape == () and float(s) == float(st) and float(z) == float(zt)
+    assert np.array_equal(xq, xq_t.float().numpy())
+    assert len(np.unique(xq)) == L + 1
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+def test_rope_matches_the_reference_op_sequence_on_torch_cpu(dtype):
+    rng = np.random.default_rng(3)
+    x = O.round_to(rng.standard_normal((2, 5, 7, 128)).astype(np.float32) * 3, dtype)
+    ang = rng.uniform(0, 6.3, size=(2, 1, 7, 64)).astype(np.float32)
+    ang = np.concatenate([ang, ang], -1)
+    cos, sin = O.round_to(np.cos(ang), dtype), O.round_to(np.sin(ang), dtype)
+    got = O.rope(x, cos, sin, dtype)
+    want = reference_rope_sequence(_t(x, dtype), _t(cos, dtype), _t(sin, dtype)).float().numpy()
+    assert np.array_equal(got, want)
+    # the two-rounding form (x*cos) + (rotate_half(x)*sin) is a different function: a restatement
+    # that rounded the second product would fail the comparison above
+    xt, ct, st_ = _t(x, dtype), _t(cos, dtype), _t(sin, dtype)
+    two = (xt * ct + torch.cat((-xt[..., 64:], xt[..., :64]), -1) * st_).float().numpy()
+    frac = np.mean(two != want)
+    assert 0.02 < frac < 0.6, frac
+    # rotation by angle 0 is the identity, by pi/2 it is rotate_half (cos, sin exactly 1 / 0)
+    one, zero = np.ones_like(cos), np.zeros_like(cos)
+    assert np.array_equal(O.rope(x, one, zero, dtype), x)
+    assert np.array_equal(O.rope(x, zero, one, dtype), np.concatenate([-x[..., 64:], x[..., :64]], -1))
 
 
 def test_quant_reciprocal_rule_differs_only_by_rounding():
@@ -311,6 +351,27 @@ def test_kivi_pack_little_endian_and_pv(bits):
     p = rng.random((1, 2, 9)).astype(np.float32)
     out = O.kivi_pv(p, words, s, mn, 32, bits)
     assert np.allclose(out, np.einsum("bht,bhtd->bhd", p, deq), atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("bits", [1, 2])
+def test_kivi_quantiser_matches_torch_eager_chain(bits, dtype):
+    """The per-token quantiser against the torch ops of qjl/new_pack.py:64-72 on a real 16-bit CPU
+    tensor (min / max per group, `(mx - mn) / L`, `data - mn`, `div_`, `clamp_`, `round_`); the
+    CPU kernel divides by the python scalar, hence levels_division="true" on the oracle side."""
+    rng = np.random.default_rng(21)
+    v = O.round_to(rng.standard_normal((2, 3, 37, 128)).astype(np.float32) * 2, dtype)
+    words, s, mn = O.kivi_quantize_pack(v, 32, bits, dtype, levels_division="true")
+    vt = _t(v, dtype).reshape(2 * 3 * 37, 4, 32)
+    mn_t, mx_t = vt.amin(-1), vt.amax(-1)
+    L = 2 ** bits - 1
+    sc_t = (mx_t - mn_t) / L
+    d = vt - mn_t.unsqueeze(-1)
+    d.div_(sc_t.unsqueeze(-1))
+    d = d.clamp_(0, L).round_().to(torch.int32)
+    assert np.array_equal(s.reshape(-1, 4), sc_t.float().numpy())
+    assert np.array_equal(mn.reshape(-1, 4), mn_t.float().numpy())
+    assert np.array_equal(O.kivi_unpack(words, bits).reshape(-1, 4, 32), d.numpy())
 
 
 def test_kivi_one_bit_words_are_packbits_little():

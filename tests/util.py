@@ -43,3 +43,18 @@ def case_to_gpu(c, dtype):
     g["ck"] = torch.from_numpy(c["ck"]).cuda()
     g["cv"] = torch.from_numpy(c["cv"]).cuda()
     return g
+
+
+def reference_rope_sequence(x, cos, sin):
+    """The torch ops that run at patch_internvl.py:125-128 of the reference (with its rotate_half,
+    :110-115, which negates the upper half of its argument in place), on a private copy of x:
+    `copy_().mul_(cos)`, in-place `rotate_half`, `addcmul_(tmp, sin)`.  cos / sin broadcast against x."""
+    x = x.clone()
+    e = torch.empty_like(x)
+    e.copy_(x).mul_(cos)
+    x1 = x[..., : x.shape[-1] // 2]
+    x2 = x[..., x.shape[-1] // 2:]
+    x2.neg_()
+    tmp = torch.cat((x2, x1), dim=-1)
+    e.addcmul_(tmp, sin)
+    return e
