@@ -57,16 +57,28 @@ def rotate_half(x):
     return torch.cat((-x[..., h:], x[..., :h]), dim=-1)
 
 
+def _rope_one(x, cos, sin):
+    # rnd(x * cos), then the fp32 sum with the exact fp32 product rotate_half(x) * sin, rounded once
+    return torch.add((x * cos).float(), rotate_half(x).float() * sin.float()).to(x.dtype)
+
+
 def apply_rotary_pos_emb(q, k, cos, sin, position_ids, unsqueeze_dim=1):
     """Rotary position embedding of q and k with the rounding of the ops the reference runs
-    (patch_internvl.py:125-128, 131-134): `x * cos` is rounded to the storage dtype, then
-    `addcmul` adds `rotate_half(x) * sin` in fp32 and rounds the sum once.  (The two-rounding
-    form `(x * cos) + (rotate_half(x) * sin)` is the commented-out line :123 and differs from
-    this by one unit in the last place in about a quarter of the elements.)  The inputs are
-    left untouched; the reference's `rotate_half` negates the upper half of its argument in place."""
+    (patch_internvl.py:125-128, 131-134): `copy_().mul_(cos)` rounds `x * cos` to the storage
+    dtype, then `addcmul_(rotate_half(x), sin)` adds the product in fp32 and rounds the sum once.
+    (The two-rounding form `(x * cos) + (rotate_half(x) * sin)` is the commented-out line :123 and
+    differs from this by one unit in the last place in about a quarter of the elements.)
+
+    The sum is written out as separate fp32 ops instead of calling `addcmul`: the device kernel the
+    reference ran rounds the fp32 sum to fp32 and then to the storage dtype, and so do these ops
+    and `cq_rope_append`; torch-ROCm's own `addcmul` on strided fp16 operands is compiled to a
+    mixed-precision multiply-add that rounds the exact sum once, which differs in about 7 of a
+    million fp16 elements (the fp32 sum lands exactly between two fp16 values).
+    The inputs are left untouched; the reference's `rotate_half` negates the upper half of its
+    argument in place."""
     cos = cos[position_ids].unsqueeze(unsqueeze_dim)
     sin = sin[position_ids].unsqueeze(unsqueeze_dim)
-    return torch.addcmul(q * cos, rotate_half(q), sin), torch.addcmul(k * cos, rotate_half(k), sin)
+    return _rope_one(q, cos, sin), _rope_one(k, cos, sin)
 
 
 @torch.no_grad()

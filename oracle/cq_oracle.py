@@ -452,8 +452,10 @@ def rope(x, cos, sin, dtype: str = "bf16") -> np.ndarray:
         e.addcmul_(tmp, sin)                         -> rnd(e + tmp * sin)
     where addcmul works in fp32 and rounds once: the product tmp * sin of two
     16-bit values is exact in fp32, the fp32 sum is rounded to fp32 and then
-    to the storage dtype.  (The commented-out line :123 would round the second
-    product to the storage dtype as well.)"""
+    to the storage dtype - the arithmetic of the device kernel the reference
+    ran (`a + alpha * (b * c)` in fp32, then the cast) and of torch's CPU
+    kernel.  (The commented-out line :123 would round the second product to
+    the storage dtype as well.)"""
     x = _f32(x)
     cos, sin = _f32(cos), _f32(sin)
     h = x.shape[-1] // 2

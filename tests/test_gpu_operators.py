@@ -164,18 +164,25 @@ def test_rope_append_equals_the_torch_op_chain_bit_for_bit(dtype, heads):
     q = v5[..., :G, :].reshape(B, 1, Hq, D).transpose(1, 2)
     k = v5[..., -2, :].transpose(1, 2)
     v = v5[..., -1, :].transpose(1, 2)
-    # (1) torch-ROCm running the reference's own op sequence on the device, (2) the oracle, (3) the
-    # package's Python helper: all four agree bit for bit
+    # (1) the oracle, (2) the package's Python helper, (3) torch-ROCm running the reference's own op
+    # sequence on the device.  (1) and (2) agree with the kernel bit for bit.  (3) does so in bf16; in
+    # fp16 torch-ROCm's addcmul on strided operands rounds the exact sum once where the kernel the
+    # reference ran rounds the fp32 sum (about 7 elements in a million sit on such a tie).
     c1, s1 = cos[pos].unsqueeze(1), sin[pos].unsqueeze(1)
-    qr, kr = reference_rope_sequence(q, c1, s1), reference_rope_sequence(k, c1, s1)
-    assert torch.equal(q_out, qr[:, :, 0])
-    assert torch.equal(kwin[:, :, 17], kr[:, :, 0]) and torch.equal(vwin[:, :, 17], v[:, :, 0])
     name = "bf16" if dtype == torch.bfloat16 else "fp16"
     assert np.array_equal(to_np(q_out), O.rope(to_np(q[:, :, 0]), to_np(c1[:, 0]), to_np(s1[:, 0]), name))
+    assert np.array_equal(to_np(kwin[:, :, 17]), O.rope(to_np(k[:, :, 0]), to_np(c1[:, 0]), to_np(s1[:, 0]), name))
+    assert torch.equal(vwin[:, :, 17], v[:, :, 0])
     qh, kh = pi.apply_rotary_pos_emb(q, k, cos, sin, pos)
-    assert torch.equal(qh, qr) and torch.equal(kh, kr)
+    assert torch.equal(qh[:, :, 0], q_out) and torch.equal(kh[:, :, 0], kwin[:, :, 17])
+    qr, kr = reference_rope_sequence(q, c1, s1), reference_rope_sequence(k, c1, s1)
+    if dtype == torch.bfloat16:
+        assert torch.equal(q_out, qr[:, :, 0]) and torch.equal(kwin[:, :, 17], kr[:, :, 0])
+    else:
+        assert (q_out != qr[:, :, 0]).float().mean().item() < 1e-3
+        assert torch.allclose(q_out.float(), qr[:, :, 0].float(), rtol=2e-3, atol=0)
     two = q * c1 + pi.rotate_half(q) * s1              # the two-rounding form is a different function
-    assert not torch.equal(two, qr)
+    assert (two != qr).float().mean().item() > 0.02
     kwin[:, :, 17] = 0
     vwin[:, :, 17] = 0
     assert not kwin.any() and not vwin.any()          # nothing else was written
@@ -209,7 +216,8 @@ def test_rope_append_full_batch_and_replay_by_device_counters():
         q = v5[..., :G, :].reshape(B, 1, Hq, D).transpose(1, 2)
         c1, s1 = cos[pos].unsqueeze(1), sin[pos].unsqueeze(1)
         qr, kr = reference_rope_sequence(q, c1, s1), reference_rope_sequence(v5[..., -2, :].transpose(1, 2), c1, s1)
-        assert torch.equal(q_out, qr[:, :, 0]) and torch.equal(kwin[:, :, step], kr[:, :, 0])
+        assert torch.equal(q_out, qr[:, :, 0]) and torch.equal(kwin[:, :, step], kr[:, :, 0])     # bf16
+        assert np.array_equal(to_np(q_out), O.rope(to_np(q[:, :, 0]), to_np(c1[:, 0]), to_np(s1[:, 0]), "bf16"))
         assert torch.equal(vwin[:, :, step], v5[:, 0, :, -1, :])
         pos.add_(1)
         row.add_(1)
