@@ -16,7 +16,8 @@ SYMBOLS = (
     "cq_version", "cq_strerror", "cq_last_hip_error",
     "cq_quantize_pack_workspace", "cq_quantize_pack", "cq_quant", "cq_quant_tensor", "cq_encode",
     "cq_lut_vecmat_qk", "cq_lut_vecmat_pv",
-    "cq_decode_attn_workspace", "cq_decode_attn", "cq_decode_attn_plan", "cq_rope_append", "cq_quantize_pack_token",
+    "cq_decode_attn_workspace", "cq_decode_attn", "cq_decode_attn_static", "cq_decode_attn_static_limit",
+    "cq_decode_attn_plan", "cq_rope_append", "cq_quantize_pack_token",
 )
 
 
@@ -91,6 +92,10 @@ def load() -> C.CDLL:
     lib.cq_decode_attn_plan.argtypes = [C.POINTER(DecodeArgs), C.POINTER(DecodePlan)]
     lib.cq_decode_attn.restype = i
     lib.cq_decode_attn.argtypes = [C.POINTER(DecodeArgs), vp]
+    lib.cq_decode_attn_static.restype = i
+    lib.cq_decode_attn_static.argtypes = [C.POINTER(DecodeArgs), vp]
+    lib.cq_decode_attn_static_limit.restype = sz
+    lib.cq_decode_attn_static_limit.argtypes = []
     lib.cq_quantize_pack_token.restype = i
     lib.cq_quantize_pack_token.argtypes = [vp, i, i, i, i, i, i64, i64, i64, i, i, vp, vp, vp, vp]
     lib.cq_rope_append.restype = i

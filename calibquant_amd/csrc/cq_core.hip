@@ -7,7 +7,7 @@ thread_local int g_last_hip_error = 0;
 
 extern "C" {
 
-int cq_version(void) { return 102; }   // 102: lut_len argument of the look-up vec-mats, cq_quant_tensor
+int cq_version(void) { return 103; }   // 103: cq_decode_attn_static; 102: lut_len argument of the look-up vec-mats, cq_quant_tensor
 
 const char* cq_strerror(int status) {
     switch (status) {
@@ -19,6 +19,7 @@ const char* cq_strerror(int status) {
         case CQ_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
         case CQ_ERR_LAUNCH: return "HIP runtime error (see cq_last_hip_error)";
         case CQ_ERR_UNSUPPORTED: return "request not covered by this build";
+        case CQ_ERR_SCRATCH_LIMIT: return "request needs more scratch than the library's static device buffer holds (cq_decode_attn_static_limit)";
         default: return "unknown status";
     }
 }

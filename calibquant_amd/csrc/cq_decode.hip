@@ -1340,6 +1340,81 @@ static int dispatch(const DecodeGeom& g, const Plan& p, int bits, hipStream_t st
     return launch<2, 1, DT, VTOK>(g, p, st);
 }
 
+// ---- static scratch for callers that cannot allocate --------------------------------------------
+// The chunked path's workspace (per-chunk logit min / max, flash-decoding partials) in a file-scope
+// device array: every GPU the library runs on holds its own copy, at its own address, until the
+// process ends.  Host code never uses the array's name as an address: the device address is asked
+// for once per device (with that device current) and kept.
+constexpr size_t kScratchBytes = static_cast<size_t>(8) << 20;
+// (`used`: no kernel names the array - they get its address as an argument - so nothing else keeps it in the code object)
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+static int scratch_address(void** out) {
+    int dev = 0;
+    CQ_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return CQ_ERR_UNSUPPORTED;
+    void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        CQ_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return CQ_ERR_LAUNCH;
+        g_scratch_ptr[dev].store(p, std::memory_order_release);   // every caller on this device gets the same address
+    }
+    *out = p;
+    return CQ_OK;
+}
+
+static int decode_entry(const cq_decode_args* a, void* workspace, size_t workspace_bytes, bool static_scratch,
+                        cq_stream_t stream) {
+    Plan p;
+    int rc = make_plan(a, &p);
+    if (rc != CQ_OK) return rc;
+    if (!a->q || !a->out) return CQ_ERR_NULL;
+    if (a->T > 0 && (!a->codes_k || !a->codes_v || !a->k_scale || !a->k_zero || !a->v_scale || !a->v_zero))
+        return CQ_ERR_NULL;
+    if (a->R > 0 && (!a->k_res || !a->v_res)) return CQ_ERR_NULL;
+    if (a->r_dev && a->mask) return CQ_ERR_UNSUPPORTED;   // the mask's length would have to follow the count
+    if (a->r_dev && (reinterpret_cast<uintptr_t>(a->r_dev) & 3)) return CQ_ERR_ALIGN;
+    if (a->T > 0 && (!aligned16(a->codes_k) || !aligned16(a->codes_v))) return CQ_ERR_ALIGN;
+    if (a->R > 0 && (!aligned16(a->k_res) || !aligned16(a->v_res) || (a->res_stride_b % 8) ||
+                     (a->res_stride_h % 8) || (a->res_stride_r % 8)))
+        return CQ_ERR_ALIGN;
+    const size_t need = p.ws_mm + p.ws_part;
+    if (static_scratch) {
+        if (need > kScratchBytes) return CQ_ERR_SCRATCH_LIMIT;
+        workspace = nullptr;
+        if (need) {
+            rc = scratch_address(&workspace);
+            if (rc != CQ_OK) return rc;
+        }
+    } else if (need && (!workspace || workspace_bytes < need || !aligned16(workspace))) {
+        return CQ_ERR_WORKSPACE;
+    }
+
+    DecodeGeom g;
+    g.q = a->q; g.ck = a->codes_k; g.cv = a->codes_v;
+    g.ks = a->k_scale; g.kz = a->k_zero; g.vs = a->v_scale; g.vz = a->v_zero;
+    g.kres = a->k_res; g.vres = a->v_res;
+    g.rs_b = a->res_stride_b; g.rs_h = a->res_stride_h; g.rs_r = a->res_stride_r;
+    g.mask = a->mask; g.mask_sb = a->mask_stride_b;
+    g.r_dev = a->r_dev;
+    g.out = a->out;
+    g.mm = static_cast<float*>(workspace);
+    g.part = need ? reinterpret_cast<float*>(static_cast<char*>(workspace) + p.ws_mm) : nullptr;
+    g.B = a->B; g.Hq = a->Hq; g.Hkv = a->Hkv; g.T = a->T; g.R = a->R; g.S = a->sprompt_len;
+    g.nsplit = p.nsplit; g.chunk = p.chunk; g.nx = p.nx;
+    g.calib = a->calibrate; g.off_max = a->calib_off_max; g.off_min = a->calib_off_min;
+    g.cap = p.cap;
+    g.one = 1.0f;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool vtok = a->v_mode == CQ_V_PER_TOKEN;
+    if (a->dtype == CQ_BF16)
+        return vtok ? dispatch<BF16, true>(g, p, a->bits, st) : dispatch<BF16, false>(g, p, a->bits, st);
+    return vtok ? dispatch<FP16, true>(g, p, a->bits, st) : dispatch<FP16, false>(g, p, a->bits, st);
+}
+
 }  // namespace cq
 
 extern "C" {
@@ -1366,42 +1441,15 @@ int cq_decode_attn_plan(const cq_decode_args* args, cq_decode_plan* plan) {
 }
 
 int cq_decode_attn(const cq_decode_args* a, cq_stream_t stream) {
-    cq::Plan p;
-    int rc = cq::make_plan(a, &p);
-    if (rc != CQ_OK) return rc;
-    if (!a->q || !a->out) return CQ_ERR_NULL;
-    if (a->T > 0 && (!a->codes_k || !a->codes_v || !a->k_scale || !a->k_zero || !a->v_scale || !a->v_zero))
-        return CQ_ERR_NULL;
-    if (a->R > 0 && (!a->k_res || !a->v_res)) return CQ_ERR_NULL;
-    if (a->r_dev && a->mask) return CQ_ERR_UNSUPPORTED;   // the mask's length would have to follow the count
-    if (a->r_dev && (reinterpret_cast<uintptr_t>(a->r_dev) & 3)) return CQ_ERR_ALIGN;
-    if (a->T > 0 && (!cq::aligned16(a->codes_k) || !cq::aligned16(a->codes_v))) return CQ_ERR_ALIGN;
-    if (a->R > 0 && (!cq::aligned16(a->k_res) || !cq::aligned16(a->v_res) || (a->res_stride_b % 8) ||
-                     (a->res_stride_h % 8) || (a->res_stride_r % 8)))
-        return CQ_ERR_ALIGN;
-    const size_t need = p.ws_mm + p.ws_part;
-    if (need && (!a->workspace || a->workspace_bytes < need || !cq::aligned16(a->workspace))) return CQ_ERR_WORKSPACE;
+    if (!a) return CQ_ERR_NULL;
+    return cq::decode_entry(a, a->workspace, a->workspace_bytes, false, stream);
+}
 
-    cq::DecodeGeom g;
-    g.q = a->q; g.ck = a->codes_k; g.cv = a->codes_v;
-    g.ks = a->k_scale; g.kz = a->k_zero; g.vs = a->v_scale; g.vz = a->v_zero;
-    g.kres = a->k_res; g.vres = a->v_res;
-    g.rs_b = a->res_stride_b; g.rs_h = a->res_stride_h; g.rs_r = a->res_stride_r;
-    g.mask = a->mask; g.mask_sb = a->mask_stride_b;
-    g.r_dev = a->r_dev;
-    g.out = a->out;
-    g.mm = static_cast<float*>(a->workspace);
-    g.part = need ? reinterpret_cast<float*>(static_cast<char*>(a->workspace) + p.ws_mm) : nullptr;
-    g.B = a->B; g.Hq = a->Hq; g.Hkv = a->Hkv; g.T = a->T; g.R = a->R; g.S = a->sprompt_len;
-    g.nsplit = p.nsplit; g.chunk = p.chunk; g.nx = p.nx;
-    g.calib = a->calibrate; g.off_max = a->calib_off_max; g.off_min = a->calib_off_min;
-    g.cap = p.cap;
-    g.one = 1.0f;
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    const bool vtok = a->v_mode == CQ_V_PER_TOKEN;
-    if (a->dtype == CQ_BF16)
-        return vtok ? cq::dispatch<cq::BF16, true>(g, p, a->bits, st) : cq::dispatch<cq::BF16, false>(g, p, a->bits, st);
-    return vtok ? cq::dispatch<cq::FP16, true>(g, p, a->bits, st) : cq::dispatch<cq::FP16, false>(g, p, a->bits, st);
+size_t cq_decode_attn_static_limit(void) { return cq::kScratchBytes; }
+
+int cq_decode_attn_static(const cq_decode_args* a, cq_stream_t stream) {
+    if (!a) return CQ_ERR_NULL;
+    return cq::decode_entry(a, nullptr, 0, true, stream);
 }
 
 }  // extern "C"

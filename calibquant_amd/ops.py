@@ -173,7 +173,7 @@ class DecodeCall:
 
     def __init__(self, q, codes_k, codes_v, k_scale, k_zero, v_scale, v_zero, k_res, v_res,
                  sprompt_len=0, bits=1, calibrate=True, calib_off_max=-3.0, calib_off_min=0.0,
-                 mask=None, out=None, force_splits=0, r_dev=None, v_mode="channel"):
+                 mask=None, out=None, force_splits=0, r_dev=None, v_mode="channel", static_scratch=False):
         _need_gpu(q, "q")
         dt = _storage_dtype(q, "q")
         if q.dim() != 3:
@@ -248,7 +248,10 @@ class DecodeCall:
             a.r_dev = r_dev.data_ptr()
             keep.append(r_dev)
         self._lib = _lib.load()
-        ws = _workspace(self._lib.cq_decode_attn_workspace(C.byref(a)), q.device)
+        # static_scratch: `cq_decode_attn_static`, whose scratch is a static device buffer inside the
+        # library - no workspace tensor, nothing allocated per call; calls on one GPU must not overlap
+        self._entry = self._lib.cq_decode_attn_static if static_scratch else self._lib.cq_decode_attn
+        ws = None if static_scratch else _workspace(self._lib.cq_decode_attn_workspace(C.byref(a)), q.device)
         if ws is not None:
             a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
             keep.append(ws)
@@ -275,7 +278,7 @@ class DecodeCall:
         return self.run()
 
     def run(self) -> torch.Tensor:
-        rc = self._lib.cq_decode_attn(self._ref, torch.cuda.current_stream(self.device).cuda_stream)
+        rc = self._entry(self._ref, torch.cuda.current_stream(self.device).cuda_stream)
         if rc:
             _lib.check(rc, "cq_decode_attn")
         return self.out

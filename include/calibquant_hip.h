@@ -36,7 +36,8 @@ enum cq_status {
     CQ_ERR_ALIGN = -4,       /* pointer or stride not 16-byte aligned */
     CQ_ERR_WORKSPACE = -5,   /* workspace missing or too small */
     CQ_ERR_LAUNCH = -6,      /* the HIP runtime reported an error */
-    CQ_ERR_UNSUPPORTED = -7  /* valid request that this build does not cover */
+    CQ_ERR_UNSUPPORTED = -7, /* valid request that this build does not cover */
+    CQ_ERR_SCRATCH_LIMIT = -8 /* cq_decode_attn_static: the request needs more scratch than the static buffer holds */
 };
 
 int cq_version(void);
@@ -199,6 +200,27 @@ typedef struct cq_decode_args {
 
 size_t cq_decode_attn_workspace(const cq_decode_args* args);
 int cq_decode_attn(const cq_decode_args* args, cq_stream_t stream);
+
+/* cq_decode_attn for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * It has no counterpart in the reference, whose operators allocate their
+ * outputs and temporaries with torch on every call.  Same arguments and the
+ * same kernels as cq_decode_attn, except that args->workspace /
+ * workspace_bytes are ignored: the scratch of the chunked path (per-chunk
+ * logit min / max and the flash-decoding partials, what
+ * cq_decode_attn_workspace() sizes) lives in a static device array of
+ * cq_decode_attn_static_limit() bytes (8 MiB) inside the library; every GPU
+ * the library runs on holds its own copy until the process ends.  A request
+ * whose plan needs more returns CQ_ERR_SCRATCH_LIMIT and launches nothing
+ * (batch 8 x 32 768 tokens needs 1.2 MiB).  The call allocates and frees
+ * nothing and does not synchronise.  Nothing in the scratch has to start at
+ * zero: every word a launch reads was written by an earlier launch of the
+ * same call.  All calls on one GPU share that GPU's array, so two calls that
+ * may overlap on one GPU (different streams, or one stream per host thread)
+ * race on it: keep them on one stream, or give the overlapping ones
+ * cq_decode_attn with workspaces of their own. */
+size_t cq_decode_attn_static_limit(void);
+int cq_decode_attn_static(const cq_decode_args* args, cq_stream_t stream);
 
 /* What cq_decode_attn would launch for these arguments (pointers are not
  * looked at; nothing is launched - the only device call is a query of the
