@@ -12,6 +12,12 @@ Prints ONE JSON line.  `value` is the
 average duration of one layer call in microseconds; `roofline` prices the
 algorithmic bytes of that call against the 8 TB/s HBM peak; `cpu_baseline` is
 the C port of the oracle timed on this host's cores on a bounded sample.
+
+Before the W warm-up steps the same calls run untimed for `--settle-ms`
+(default 300 ms): the device takes that long under this load to reach its
+steady state (a run of 20 steps straight after the inputs are built reads
+about 10 % slower than one of 4 000), and the steady state is what a decode
+loop of thousands of layer calls per second sees.  `config.settle_ms` states it.
 """
 from __future__ import annotations
 
@@ -85,7 +91,24 @@ def build_sets(torch, ops, shape, bits, nsets, seed):
     return sets
 
 
-def time_calls(torch, calls, steps, warmup):
+def settle(torch, run, ms):
+    """Run `run(i)` untimed for about `ms` milliseconds of device time."""
+    if ms <= 0:
+        return
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(8):
+        run(i)
+    end.record()
+    torch.cuda.synchronize()
+    per = max(start.elapsed_time(end) / 8, 1e-3)
+    for i in range(int(ms / per)):
+        run(i)
+    torch.cuda.synchronize()
+
+
+def time_calls(torch, calls, steps, warmup, settle_ms=0.0):
+    settle(torch, lambda i: calls[i % len(calls)].run(), settle_ms)
     for i in range(warmup):
         calls[i % len(calls)].run()
     torch.cuda.synchronize()
@@ -161,7 +184,27 @@ def _time_fn(torch, fn, steps, warmup):
     return start.elapsed_time(end) / steps
 
 
-def side_legs(torch, ops, shape, bits, sets):
+def prefill_leg(torch, ops, shape, bits, steps=40, warmup=10, contiguous=False):
+    """Prefill quantise-and-pack of one K tensor of the layer shape: read as the strided key block of
+    a fused projection output (what the attention forward hands over), or as a contiguous (B, T, H, D)
+    tensor; priced against the read-once roofline."""
+    B, Hq, Hkv, D, T, R, S = shape
+    dev = torch.device("cuda:0")
+    G = Hq // Hkv
+    if contiguous:
+        k_view = torch.randn((B, T, Hkv, D), device=dev, dtype=torch.bfloat16)
+    else:
+        proj = torch.randn((B, T, Hkv, G + 2, D), device=dev, dtype=torch.bfloat16)
+        k_view = proj[..., -2, :]
+    clip = 0.5 if bits == 1 else 1.0
+    ms = _time_fn(torch, lambda: ops.quantize_pack(k_view, bits, clip), steps, warmup)
+    rd = B * T * Hkv * D * 2 + B * Hkv * T * D * bits // 8
+    return {"us_per_tensor": round(ms * 1e3, 1), "algorithmic_bytes": rd, "achieved_GBps": round(rd / ms / 1e6, 1),
+            "frac_of_hbm_peak": round(rd / ms / 1e6 / HBM_PEAK_GBPS, 4), "bits": bits,
+            "input": "contiguous (B, T, H, D)" if contiguous else "key block of the fused projection output"}
+
+
+def side_legs(torch, ops, shape, bits, sets, settle_ms=0.0, only_token=False):
     """Figures next to the headline one, same layer shape: the prefill quantise-and-pack of one
     K tensor read as the strided key block of a fused projection output (read-once roofline),
     and the decode kernel on per-token values (`v_mode = token`)."""
@@ -169,37 +212,41 @@ def side_legs(torch, ops, shape, bits, sets):
     dev = torch.device("cuda:0")
     G = Hq // Hkv
     res = {}
+    if not only_token:
+        res["prefill_quantize_pack"] = prefill_leg(torch, ops, shape, bits)
     proj = torch.randn((B, T, Hkv, G + 2, D), device=dev, dtype=torch.bfloat16)
     k_view, v_view = proj[..., -2, :], proj[..., -1, :]
-    clip = 0.5 if bits == 1 else 1.0
-    ms = _time_fn(torch, lambda: ops.quantize_pack(k_view, bits, clip), 10, 3)
-    rd = B * T * Hkv * D * 2 + B * Hkv * T * D * bits // 8
-    res["prefill_quantize_pack"] = {"us_per_tensor": round(ms * 1e3, 1), "algorithmic_bytes": rd,
-                                    "achieved_GBps": round(rd / ms / 1e6, 1),
-                                    "frac_of_hbm_peak": round(rd / ms / 1e6 / HBM_PEAK_GBPS, 4)}
     ms_t = _time_fn(torch, lambda: ops.quantize_pack_token(v_view, bits), 10, 3)
-    words, vsc, vmn = ops.quantize_pack_token(v_view, bits)
+    # per-token values: every buffer set gets values of its own, so the calls rotate over as many
+    # distinct code buffers as the headline measurement does
+    calls = []
+    for i, x in enumerate(sets):
+        vv = torch.randn((B, T, Hkv, D), device=dev, dtype=torch.bfloat16)
+        words, vsc, vmn = ops.quantize_pack_token(vv, bits)
+        del vv
+        calls.append(ops.DecodeCall(x["q"], x["ck"], words, x["sk"], x["zk"], vsc, vmn, x["kr"], x["vr"],
+                                    sprompt_len=S, bits=bits, v_mode="token"))
     del proj, k_view, v_view
-    s0 = sets[0]
-    call = ops.DecodeCall(s0["q"], s0["ck"], words, s0["sk"], s0["zk"], vsc, vmn, s0["kr"], s0["vr"],
-                          sprompt_len=S, bits=bits, v_mode="token")
-    ms_d = _time_fn(torch, call.run, 100, 10)
+    ms_d = time_calls(torch, calls, 200, 20, settle_ms)
     nb = algorithmic_bytes(B, Hq, Hkv, D, T, R, bits) - 2 * B * Hkv * D * 2 + 2 * B * Hkv * T * (D // 32) * 2
     res["per_token_values"] = {"quantize_pack_token_us": round(ms_t * 1e3, 1), "decode_us_layer": round(ms_d * 1e3, 2),
                                "algorithmic_bytes": nb, "achieved_GBps": round(nb / ms_d / 1e6, 1),
-                               "note": "one buffer set (codes may be served from the Infinity Cache)"}
-    del words, vsc, vmn, call
+                               "frac_of_hbm_peak": round(nb / ms_d / 1e6 / HBM_PEAK_GBPS, 4),
+                               "launch_plan": calls[0].plan(), "note": f"{len(calls)} buffer sets"}
+    del calls
+    if only_token:
+        return res
     # the other bit width of the same layer shape (BASELINE's layer configuration names b = 1 and b = 2)
     ob = 2 if bits == 1 else 1
-    osets = build_sets(torch, ops, shape, ob, 2, 4321)
+    osets = build_sets(torch, ops, shape, ob, 2 if ob == 2 else len(sets), 4321)
     ocalls = [ops.DecodeCall(x["q"], x["ck"], x["cv"], x["sk"], x["zk"], x["sv"], x["zv"], x["kr"], x["vr"],
                              sprompt_len=S, bits=ob) for x in osets]
-    ms_o = time_calls(torch, ocalls, 100, 10)
+    ms_o = time_calls(torch, ocalls, 200, 20, settle_ms)
     nbo = algorithmic_bytes(B, Hq, Hkv, D, T, R, ob)
     res[f"decode_{ob}bit"] = {"us_layer": round(ms_o * 1e3, 2), "algorithmic_bytes": nbo,
                               "achieved_GBps": round(nbo / ms_o / 1e6, 1),
                               "frac_of_hbm_peak": round(nbo / ms_o / 1e6 / HBM_PEAK_GBPS, 4),
-                              "launch_plan": ocalls[0].plan(), "note": "two buffer sets"}
+                              "launch_plan": ocalls[0].plan(), "note": f"{len(osets)} buffer sets"}
     return res
 
 
@@ -230,6 +277,39 @@ def cpu_baseline(torch, sets, shape, bits, budget_s=12.0):
     return {"value": round(med * 1e6 * B / bs, 1), "unit": "us/layer", "cores": cores, "kind": "port",
             "sample": f"oracle/cq_oracle.c (OpenMP) on {bs} of {B} batch rows, median of {reps} runs, "
                       f"scaled x{B // bs} to the full batch"}
+
+
+def cpu_reference_config(torch, ops, seed=1234):
+    """The CPU-runnable reference configuration, CPU and GPU side by side: batch 1, 32 query / 8 KV
+    heads, head_dim 128, 1 024 tokens, fp16, K / V ~ N(0,1) with four key channels per kv-head scaled
+    x10, 1-bit codes (clip 0.5 / 0.3), calibration offsets (-3, 0), no window.  The C port of the
+    oracle on the host cores and the HIP path on the GPU run on the same packed state."""
+    import numpy as np
+    from oracle import c_port, cq_oracle as O
+    B, Hq, Hkv, D, T = 1, 32, 8, 128, 1024
+    k, v = O.synth_kv(B, T, Hkv, D, "fp16", seed=seed, outliers=4, outlier_kind="x10")
+    q = O.round_to(np.random.default_rng(seed + 1).standard_normal((B, Hq, D), dtype=np.float32), "fp16")
+    g = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(torch.float16).cuda()  # noqa: E731
+    ck, sk, zk = ops.quantize_pack(g(k), 1, 0.5)
+    cv, sv, zv = ops.quantize_pack(g(v), 1, 0.3)
+    call = ops.DecodeCall(g(q), ck, cv, sk, zk, sv, zv, None, None, sprompt_len=0, bits=1)
+    gpu_ms = _time_fn(torch, call.run, 200, 20)
+    out = call.run().float().cpu().numpy()
+    f = lambda t: t.float().cpu().numpy()  # noqa: E731
+    args = (q, ck.cpu().numpy(), cv.cpu().numpy(), f(sk), f(zk), f(sv), f(zv), None, None, 0, 1)
+    c_port.build()
+    want = c_port.decode_attention(*args)
+    times = []
+    for _ in range(30):
+        t0 = time.perf_counter()
+        c_port.decode_attention(*args)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    err = np.abs(out - want)
+    return {"workload": "cpu-reference-config-b1-kv1024-fp16", "cpu_us_layer": round(times[len(times) // 2] * 1e6, 1),
+            "gpu_us_layer": round(gpu_ms * 1e3, 2), "launch_plan": call.plan(),
+            "max_abs_gpu_vs_cpu": float(err.max()), "mean_abs_gpu_vs_cpu": float(err.mean()),
+            "sample": "whole configuration, median of 30 CPU runs"}
 
 
 def model_leg(torch, batch=64, tiles=13, sys_len=41, text_len=23, new_tokens=128, seed=1234, model_name="8b"):
@@ -371,6 +451,10 @@ def main():
     ap.add_argument("--no-side", action="store_true", help="skip the prefill / per-token-value side figures")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch three 256 MiB device copies (known traffic, for scaling profiler byte counters)")
+    ap.add_argument("--settle-ms", type=float, default=300.0,
+                    help="untimed run of the same calls before the warm-up steps, in ms of device time")
+    ap.add_argument("--only", default=None, choices=("prefill", "prefill-contiguous", "token-values"),
+                    help="run one side figure alone (for profiling it) and print its JSON")
     ap.add_argument("--seed", type=int, default=1234)
     a = ap.parse_args()
     if a.gpus != 1:
@@ -386,7 +470,13 @@ def main():
 
     shape = WORKLOADS[a.workload]
     B, Hq, Hkv, D, T, R, S = shape
+    if a.only in ("prefill", "prefill-contiguous"):
+        print(json.dumps(prefill_leg(torch, ops, shape, a.bits, a.steps, a.warmup, a.only == "prefill-contiguous")))
+        return
     sets = build_sets(torch, ops, shape, a.bits, a.sets, a.seed)
+    if a.only == "token-values":
+        print(json.dumps(side_legs(torch, ops, shape, a.bits, sets, a.settle_ms, only_token=True)))
+        return
     calls = [ops.DecodeCall(s["q"], s["ck"], s["cv"], s["sk"], s["zk"], s["sv"], s["zv"], s["kr"], s["vr"],
                             sprompt_len=S, bits=a.bits) for s in sets]
     if a.copy_calibration:
@@ -395,7 +485,7 @@ def main():
         for _ in range(3):
             dst.copy_(src)
         torch.cuda.synchronize()
-    ms = time_calls(torch, calls, a.steps, a.warmup)
+    ms = time_calls(torch, calls, a.steps, a.warmup, a.settle_ms)
     plan = calls[0].plan()
     nbytes = algorithmic_bytes(B, Hq, Hkv, D, T, R, a.bits)
     gbps = nbytes / (ms * 1e-3) / 1e9
@@ -415,7 +505,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": a.workload, "batch": B, "q_heads": Hq, "kv_heads": Hkv, "head_dim": D,
                    "kv_packed_tokens": T, "kv_residual_rows": R, "bits": a.bits, "storage_dtype": "bf16",
-                   "buffer_sets": a.sets, "launches_per_step": plan["launches"], "launch_plan": plan},
+                   "buffer_sets": a.sets, "settle_ms": a.settle_ms, "launches_per_step": plan["launches"],
+                   "launch_plan": plan},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": measured_traffic(a.workload, a.bits),
                      "algorithmic_bytes": nbytes},
@@ -433,9 +524,13 @@ def main():
             out["fp16_kv_error"] = repr(e)[:200]
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline(torch, sets, shape, a.bits)
+        try:
+            out["cpu_baseline"]["reference_config"] = cpu_reference_config(torch, ops, a.seed)
+        except Exception as e:  # must not sink the measurement
+            out["cpu_baseline"]["reference_config"] = {"error": repr(e)[:200]}
     if not a.no_side:
         try:
-            out["side_legs"] = side_legs(torch, ops, shape, a.bits, sets)
+            out["side_legs"] = side_legs(torch, ops, shape, a.bits, sets, a.settle_ms)
         except Exception as e:  # side figures must not sink the measurement
             out["side_legs"] = {"error": repr(e)[:300]}
     if not a.no_model and a.workload == DEFAULT_WORKLOAD and a.bits == 1:

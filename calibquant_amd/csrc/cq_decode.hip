@@ -72,6 +72,8 @@ struct DecodeGeom {
     int cap;      // logits capacity of the LDS layout, tokens
     FastDiv d_ng, d_nx, d_hkv;   // divisors of the unit decomposition: head groups, chunks (+ residual unit), kv heads
     int G;        // query heads per kv head
+    int ncu;      // paired launch whose workgroups are all resident from the start (at most two per compute unit):
+                  // the number of compute units (the two workgroups of a unit are told apart by it); else 0
     float one;    // 1.0f, opaque to the compiler: keeps f16 -> f32 accumulation in one mixed-precision FMA
 };
 
@@ -267,6 +269,31 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
     const int lane = tid & 63;
     const int wv = tid >> 6;
     const int G = g.G;
+    // Wave priorities of the paired launch (two 512-thread workgroups per compute unit, all of them
+    // resident from the first cycle).  Left to the hardware's own arbitration the workgroup that was
+    // dispatched first gets most of the issue slots: it ends after about 56 K cycles and the other one
+    // after 77 K, the last 20 K alone on the unit with too few waves to hide its own latencies.  With the
+    // short, latency-bound phases (set-up, table build, reductions, staging, exp) above the throughput
+    // phases, the first workgroup ahead in the K look-ups and the second ahead in the packed-V loop,
+    // both end together (measured at the benchmark shape: 36.0 -> 33.8 us, same results).  Launches with
+    // more workgroups than fit at once start their later workgroups as earlier ones end, which staggers
+    // them by itself; there the priorities are left alone (with them: 66 -> 84 us at batch 128).
+    // `second`: the workgroup that shares its unit with an older one (workgroups are handed out unit by
+    // unit, g.ncu at a time).
+    const bool prio_on = NT == 512 && g.ncu > 0;
+    const bool second = prio_on && blockIdx.x >= static_cast<unsigned>(g.ncu);
+    auto phase_priority = [&](auto phase_c) {
+        constexpr int PH = decltype(phase_c)::value;   // 0 set-up and tables, 1 K look-ups, 2 min/max .. exp, 3 packed V, 4 folds, window, merge
+        if constexpr (NT == 512) {
+            if (prio_on) {
+                if constexpr (PH == 0 || PH == 2) __builtin_amdgcn_s_setprio(2);
+                else if constexpr (PH == 1) { if (second) __builtin_amdgcn_s_setprio(0); else __builtin_amdgcn_s_setprio(1); }
+                else if constexpr (PH == 3) { if (second) __builtin_amdgcn_s_setprio(2); else __builtin_amdgcn_s_setprio(1); }
+                else __builtin_amdgcn_s_setprio(0);
+            }
+        }
+    };
+    phase_priority(std::integral_constant<int, 0>{});
 
     uint32_t vb = static_cast<uint32_t>(virtual_block_id());
     uint32_t qn = g.d_ng.quot(vb);
@@ -453,6 +480,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
         }
         __syncthreads();
 
+        phase_priority(std::integral_constant<int, 1>{});
         // ---- phase 3: logits of the chunk ------------------------------------------------
         // Lane l walks the byte positions of a pass in the order k ^ (l mod NBP): in every step
         // the lanes that the LDS serves together read NBP distinct positions of the
@@ -618,6 +646,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             k_pass(std::integral_constant<int, 3>{});
         }
     }
+    phase_priority(std::integral_constant<int, 2>{});
     if (n > 0) {   // one reduction for both: max of (-min, max)
         float mm2[2 * HPB];
 #pragma unroll
@@ -818,6 +847,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             const uint32_t wtab_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
                 (__attribute__((address_space(3))) unsigned char*)wtab));
 
+            phase_priority(std::integral_constant<int, 3>{});
             for (int vs0 = 0; vs0 < npad; vs0 += L::VSUB) {
                 const int vn = min(L::VSUB, npad - vs0);
                 if (vs0 > 0) {
@@ -907,6 +937,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                     __builtin_amdgcn_wave_barrier();
                 }
             }
+            phase_priority(std::integral_constant<int, 4>{});
             load_res_k(0, rk);   // first residual tile: in flight during the fold below
             load_res_v(0, rv);
             // per-wave partial sums of e (and of e * minimum), folded by the output threads below
@@ -1297,6 +1328,7 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
     }
     DecodeGeom gm = g;
     gm.G = G;
+    gm.ncu = (NT == 512 && static_cast<int64_t>(units) * g.nx <= 2 * static_cast<int64_t>(pair_units())) ? pair_units() : 0;
     gm.d_ng.set(static_cast<uint32_t>(ngroups(G, HPB)));
     gm.d_nx.set(static_cast<uint32_t>(g.nx));
     gm.d_hkv.set(static_cast<uint32_t>(g.Hkv));
