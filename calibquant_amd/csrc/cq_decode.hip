@@ -92,7 +92,12 @@ constexpr int cmin(int a, int b) { return a < b ? a : b; }
 template <int BITS, int HPB, bool VTOK = false, int NT_ = 1024, int REGL = 0> struct Lay {
     static constexpr int kNT = NT_;                 // threads per workgroup
     static constexpr int kNW = kNT / kWave;         // waves per workgroup
-    static constexpr int kResTile = kNT / 8;        // residual rows per tile (8 lanes per row)
+    // residual window: tiles of 128 rows for either workgroup size - a 512-thread workgroup puts 4 lanes on a
+    // row (32 channels each), a 1024-thread one 8 (16 channels each)
+    static constexpr int LPR = kNT / 128;           // lanes per residual row
+    static constexpr int kResTile = kNT / LPR;      // residual rows per tile
+    static constexpr int NKP = 16 / LPR;            // 16-byte pieces of a row per lane
+    static constexpr int RPW = kResTile / kNW;      // rows of a tile whose values one wave multiplies
     static constexpr int NB = 16 * BITS;            // bytes per packed row
     static constexpr int PC = NB * 8;               // bit lanes per row
     static constexpr int GPW = kWave / NB;          // 4-token groups per wave pass
@@ -347,26 +352,27 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
     const uint4* cvp = reinterpret_cast<const uint4*>((has_img ? g.cv : static_cast<const uint8_t*>(g.q)) + code_off);
     const U4* cvp4 = reinterpret_cast<const U4*>(cvp);
     const int last_u = has_img ? n * NB / 16 - 1 : 0;   // last valid 16-byte unit of either stream
-    // residual tile: K slice (row = tid/8, 16 elements); V: a wave owns 8 rows of the tile and a
+    // residual tile: K slice (row = tid / LPR, 128 / LPR elements); V: a wave owns RPW rows of the tile and a
     // lane one channel pair of each of them, so the value products need no fold inside the wave
-    const int l8 = tid & 7, krow = tid >> 3;
+    constexpr int LPR = L::LPR, NKP = L::NKP, RPW = L::RPW;
+    const int lq = tid % LPR, krow = tid / LPR;
     const int wvr = __builtin_amdgcn_readfirstlane(wv);   // wave-uniform: scalar row arithmetic
     const int64_t res_off = do_res ? b * g.rs_b + hkv * g.rs_h : 0;   // one offset for both windows
     const uint16_t* kb = static_cast<const uint16_t*>(do_res ? g.kres : g.q) + res_off;
     const uint16_t* vbp = static_cast<const uint16_t*>(do_res ? g.vres : g.q) + res_off;
     const int last_r = do_res ? R - 1 : 0;
     const int64_t rs_r = do_res ? g.rs_r : 0;
-    uint4 rk[2];
-    uint32_t rv[8];
+    uint4 rk[NKP];
+    uint32_t rv[RPW];
     auto load_res_k = [&](int r0, uint4* k2) {   // rows past R re-read row R-1 (their logit is masked)
-        const uint16_t* kp = kb + min(r0 + krow, last_r) * rs_r;
-        k2[0] = *reinterpret_cast<const uint4*>(kp + l8 * 8);
-        k2[1] = *reinterpret_cast<const uint4*>(kp + 64 + l8 * 8);
+        const uint16_t* kp = kb + min(r0 + krow, last_r) * rs_r + lq * 8;
+#pragma unroll
+        for (int i = 0; i < NKP; ++i) k2[i] = *reinterpret_cast<const uint4*>(kp + i * (LPR * 8));   // piece i * LPR + lq
     };
     auto load_res_v = [&](int r0, uint32_t* v8) {   // rows past R re-read row R-1 (their weight is 0)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int r2 = min(r0 + wvr * 8 + i, last_r);
+        for (int i = 0; i < RPW; ++i) {
+            const int r2 = min(r0 + wvr * RPW + i, last_r);
             v8[i] = *reinterpret_cast<const uint32_t*>(vbp + r2 * rs_r + 2 * lane);
         }
     };
@@ -938,8 +944,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                 }
             }
             phase_priority(std::integral_constant<int, 4>{});
-            load_res_k(0, rk);   // first residual tile: in flight during the fold below
-            load_res_v(0, rv);
+            load_res_k(0, rk);   // first residual tile's K rows: in flight during the fold below
             // per-wave partial sums of e (and of e * minimum), folded by the output threads below
             constexpr int kSums = VTOK ? (L::NGRP + 1) * HPB : HPB;
             wave_reduce_n<HPB>(ls, OpSum(), 0.f);
@@ -1000,10 +1005,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             __syncthreads();
         }
 
-        if (n == 0) {
-            load_res_k(0, rk);
-            load_res_v(0, rv);
-        }
+        if (n == 0) load_res_k(0, rk);
         // ---- phase 6: full-precision residual rows, online softmax.  Runs last: its first
         // tile is requested when the packed-V phase ends and arrives during that phase's fold.
 #pragma unroll
@@ -1029,20 +1031,23 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             for (int r0 = 0; r0 < R; r0 += kResTile) {
                 const bool more = r0 + kResTile < R;
                 const int r = r0 + krow;
+                load_res_v(r0, rv);   // the tile's value words: in flight while its logits and weights are worked out
                 float dot[HPB];
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) {
-                    const uint4 qa = q128[h * (kD / 8) + l8];
-                    const uint4 qb = q128[h * (kD / 8) + 8 + l8];
                     float a = 0.f;
-                    a = dot2<DT>(qa.x, rk[0].x, a); a = dot2<DT>(qa.y, rk[0].y, a);
-                    a = dot2<DT>(qa.z, rk[0].z, a); a = dot2<DT>(qa.w, rk[0].w, a);
-                    a = dot2<DT>(qb.x, rk[1].x, a); a = dot2<DT>(qb.y, rk[1].y, a);
-                    a = dot2<DT>(qb.z, rk[1].z, a); a = dot2<DT>(qb.w, rk[1].w, a);
-                    dot[h] = oct_reduce(a, OpSum(), 0.f) * inv_sqrt_d;
+#pragma unroll
+                    for (int i = 0; i < NKP; ++i) {
+                        const uint4 qa = q128[h * (kD / 8) + i * LPR + lq];
+                        a = dot2<DT>(qa.x, rk[i].x, a); a = dot2<DT>(qa.y, rk[i].y, a);
+                        a = dot2<DT>(qa.z, rk[i].z, a); a = dot2<DT>(qa.w, rk[i].w, a);
+                    }
+                    dot[h] = (LPR == 4 ? quad_reduce(a, OpSum(), 0.f) : oct_reduce(a, OpSum(), 0.f)) * inv_sqrt_d;
+                    // one head's q pieces at a time: all of them side by side would not fit the registers
+                    if constexpr (NKP > 2) __builtin_amdgcn_sched_barrier(0);
                 }
                 if (more) load_res_k(r0 + kResTile, rk);   // next tile's K slice, in place
-                if (l8 == 0) {
+                if (lq == 0) {
                     float mv = 0.f;
                     if (mk && r < R) mv = mk[r < g.S ? r : g.T + r];
 #pragma unroll
@@ -1082,16 +1087,15 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                     }
                 }
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
+                for (int i = 0; i < RPW; ++i) {
                     const float f0 = Cvt<DT>::lo(rv[i]), f1 = Cvt<DT>::hi(rv[i]);
-                    const V p = reinterpret_cast<const V*>(pres)[wvr * 8 + i];   // the row's weights (0 past R), one address per wave
+                    const V p = reinterpret_cast<const V*>(pres)[wvr * RPW + i];   // the row's weights (0 past R), one address per wave
 #pragma unroll
                     for (int h = 0; h < HPB; ++h) {
                         accv[0][h] = __builtin_fmaf(p.v[h], f0, accv[0][h]);
                         accv[1][h] = __builtin_fmaf(p.v[h], f1, accv[1][h]);
                     }
                 }
-                if (more) load_res_v(r0 + kResTile, rv);   // next tile's V words, in place
             }
             __syncthreads();
             float* red2 = reinterpret_cast<float*>(regA);  // [wave][head][kD]: the fold reads consecutive words
