@@ -314,8 +314,8 @@ def cpu_reference_config(torch, ops, seed=1234):
 
 def model_leg(torch, batch=64, tiles=13, sys_len=41, text_len=23, new_tokens=128, seed=1234, model_name="8b"):
     """InternVL2.5-8B-shaped decode (InternLM2.5-7B language model: 32 layers, hidden 4096, 32/8
-    heads, head_dim 128, vocab 92 553), random-init bf16 weights, synthetic uniform-noise tiles
-    through a stand-in vision tower: tokens/s of `new_tokens` greedy steps at `batch`, prefill
+    heads, head_dim 128, vocab 92 553; InternViT-300M-shaped vision tower), random-init bf16 weights,
+    synthetic uniform-noise tiles: tokens/s of `new_tokens` greedy steps at `batch`, prefill
     excluded, 1-bit KV (patched attention) vs full-precision KV (unpatched) on the same weights."""
     from calibquant_amd import patch_internvl as pi
     from calibquant_amd.internlm2 import InternLM2Attention, InternLM2Config, InternVLChatStandIn
@@ -325,8 +325,10 @@ def model_leg(torch, batch=64, tiles=13, sys_len=41, text_len=23, new_tokens=128
     torch.set_default_dtype(torch.bfloat16)
     try:
         with torch.device(dev):
+            from calibquant_amd.internvit import InternViTConfig
             cfg = InternLM2Config.internvl2_5_26b() if model_name == "26b" else InternLM2Config.internvl2_5_8b()
-            model = InternVLChatStandIn(cfg).eval()
+            vit = InternViTConfig.internvit_6b() if model_name == "26b" else InternViTConfig.internvit_300m()
+            model = InternVLChatStandIn(cfg, vit=vit).eval()
     finally:
         torch.set_default_dtype(prev)
     T = tiles * 256
@@ -335,7 +337,8 @@ def model_leg(torch, batch=64, tiles=13, sys_len=41, text_len=23, new_tokens=128
     ids[:, sys_len:sys_len + T] = model.img_context_token_id
     fp_forward, fp_generate = InternLM2Attention.forward, InternVLChatStandIn.generate
     res = {"model": "internvl2.5-" + model_name + "-shaped", "prompt_tokens": N, "image_tokens": T,
-           "new_tokens": new_tokens, "batch": batch}
+           "new_tokens": new_tokens, "batch": batch,
+           "vision_tower": "internvit-6b-shaped" if model_name == "26b" else "internvit-300m-shaped"}
 
     def features():
         vis = []

@@ -11,8 +11,10 @@ chat model exposes `language_model.model.layers[i].attention`,
 `extract_feature(pixel_values)` and `img_context_token_id`.  The fused wqkv
 weight uses the `(h gs d)` interleave of the reference (patch_internvl.py:219-234):
 per kv-head, `num_key_value_groups` query heads, then the key, then the value.
-The vision tower is a stand-in (patch embedding + pooling to 256 tokens per
-tile): it only feeds the prefill."""
+The vision tower is either the InternViT-shaped encoder of `internvit.py`
+(`InternVLChatStandIn(cfg, vit=InternViTConfig...)`) or, by default, a one-layer
+stand-in (patch projection to 256 tokens per tile) for tests that only need the
+shapes: either way it only feeds the prefill."""
 from __future__ import annotations
 
 import math
@@ -264,11 +266,17 @@ class StandInVisionTower(nn.Module):
 
 
 class InternVLChatStandIn(nn.Module):
-    def __init__(self, cfg: InternLM2Config, img_context_token_id: Optional[int] = None):
+    def __init__(self, cfg: InternLM2Config, img_context_token_id: Optional[int] = None, vit=None):
+        """vit: an `internvit.InternViTConfig` for the InternViT-shaped tower (encoder, pixel shuffle,
+        projector), or None for the one-layer stand-in."""
         super().__init__()
         self.config = cfg
         self.language_model = InternLM2ForCausalLM(cfg)
-        self.vision = StandInVisionTower(cfg.hidden_size)
+        if vit is None:
+            self.vision = StandInVisionTower(cfg.hidden_size)
+        else:
+            from .internvit import InternViTTower
+            self.vision = InternViTTower(vit, cfg.hidden_size)
         self.img_context_token_id = cfg.vocab_size - 1 if img_context_token_id is None else img_context_token_id
         self.num_image_token = 256
 

@@ -13,10 +13,10 @@ from tests.util import to_np
 pytestmark = pytest.mark.gpu
 
 
-def _tiny_model(layers=2, seed=0):
+def _tiny_model(layers=2, seed=0, vit=None):
     from calibquant_amd.internlm2 import InternLM2Config, InternVLChatStandIn
     torch.manual_seed(seed)
-    m = InternVLChatStandIn(InternLM2Config.tiny(layers)).cuda().to(torch.bfloat16).eval()
+    m = InternVLChatStandIn(InternLM2Config.tiny(layers), vit=vit).cuda().to(torch.bfloat16).eval()
     return m
 
 
@@ -131,13 +131,17 @@ def test_patched_model_without_image_tokens_equals_the_fp_model():
         InternLM2Attention.forward, InternVLChatStandIn.generate = fp_forward, fp_generate
 
 
-def test_patch_model_and_custom_generate_end_to_end():
-    """Two synthetic tiles per sample -> 512 image tokens, quantised at prefill, 8 greedy tokens."""
+@pytest.mark.parametrize("tower", ["stand-in", "internvit"])
+def test_patch_model_and_custom_generate_end_to_end(tower):
+    """Synthetic tiles -> 256 image tokens each, quantised at prefill, 8 greedy tokens.  With the
+    InternViT-shaped tower the 12 tiles go through `extract_feature` in two chunks (10 + 2), as the
+    reference's `custom_generate` runs them (patch_internvl.py:53-65)."""
     from calibquant_amd import patch_internvl as pi
     from calibquant_amd.internlm2 import InternLM2Attention, InternVLChatStandIn
+    from calibquant_amd.internvit import InternViTConfig
     fp_forward, fp_generate = InternLM2Attention.forward, InternVLChatStandIn.generate
-    m = _tiny_model(seed=3)
-    B, S, tiles, txt = 2, 41, 2, 9
+    m = _tiny_model(seed=3, vit=InternViTConfig.tiny() if tower == "internvit" else None)
+    B, S, tiles, txt = (2, 41, 6, 9) if tower == "internvit" else (2, 41, 2, 9)
     T = tiles * 256
     ids = torch.randint(0, 500, (B, S + T + txt), device="cuda")
     ids[:, S:S + T] = m.img_context_token_id

@@ -59,3 +59,28 @@ def test_transform_is_resize_scale_and_affine_normalisation():
     assert xg.shape == (3, 32, 32)
     px = P.load_image(Image.fromarray(rng.integers(0, 256, size=(100, 400, 3), dtype=np.uint8), "RGB"), input_size=32, max_num=6)
     assert px.shape == (4 + 1, 3, 32, 32)
+
+
+def test_internvit_shaped_tower_shapes_and_pixel_shuffle():
+    """The InternViT-shaped tower turns 448 x 448 tiles into 256 tokens of the language model's width;
+    the pixel shuffle gathers every 2 x 2 block of patches into one token, block row first."""
+    import torch
+    from calibquant_amd.internvit import InternViTConfig, InternViTTower, pixel_shuffle
+    x = torch.arange(2 * 4 * 6 * 3, dtype=torch.float32).reshape(2, 4, 6, 3)
+    y = pixel_shuffle(x, 0.5)
+    assert y.shape == (2, 2, 3, 12)
+    for n in range(2):
+        for w in range(2):
+            for h in range(3):
+                want = torch.cat([x[n, 2 * w + a, 2 * h + b] for a in range(2) for b in range(2)])
+                assert torch.equal(y[n, w, h], want)
+    torch.manual_seed(0)
+    tower = InternViTTower(InternViTConfig.tiny(), llm_hidden=96).eval()
+    with torch.no_grad():
+        out = tower(torch.rand(3, 3, 448, 448))
+    assert out.shape == (3, 256, 96) and tower.num_image_token == 256 and torch.isfinite(out).all()
+    # the 300M preset has the published size (about 0.3 billion parameters); built without storage
+    with torch.device("meta"):
+        big = InternViTTower(InternViTConfig.internvit_300m(), llm_hidden=4096)
+    enc = sum(p.numel() for n_, p in big.named_parameters() if not n_.startswith("mlp1"))
+    assert 0.29e9 < enc < 0.32e9, enc
