@@ -184,7 +184,7 @@ def _time_fn(torch, fn, steps, warmup):
     return start.elapsed_time(end) / steps
 
 
-def prefill_leg(torch, ops, shape, bits, steps=40, warmup=10, contiguous=False):
+def prefill_leg(torch, ops, shape, bits, steps=40, warmup=10, contiguous=False, rope=True):
     """Prefill quantise-and-pack of one K tensor of the layer shape: read as the strided key block of
     a fused projection output (what the attention forward hands over), or as a contiguous (B, T, H, D)
     tensor; priced against the read-once roofline."""
@@ -199,9 +199,26 @@ def prefill_leg(torch, ops, shape, bits, steps=40, warmup=10, contiguous=False):
     clip = 0.5 if bits == 1 else 1.0
     ms = _time_fn(torch, lambda: ops.quantize_pack(k_view, bits, clip), steps, warmup)
     rd = B * T * Hkv * D * 2 + B * Hkv * T * D * bits // 8
-    return {"us_per_tensor": round(ms * 1e3, 1), "algorithmic_bytes": rd, "achieved_GBps": round(rd / ms / 1e6, 1),
-            "frac_of_hbm_peak": round(rd / ms / 1e6 / HBM_PEAK_GBPS, 4), "bits": bits,
-            "input": "contiguous (B, T, H, D)" if contiguous else "key block of the fused projection output"}
+    res = {"us_per_tensor": round(ms * 1e3, 1), "algorithmic_bytes": rd, "achieved_GBps": round(rd / ms / 1e6, 1),
+           "frac_of_hbm_peak": round(rd / ms / 1e6 / HBM_PEAK_GBPS, 4), "bits": bits,
+           "input": "contiguous (B, T, H, D)" if contiguous else "key block of the fused projection output"}
+    if rope and T <= ops.ROPE_FUSED_MAX_T:
+        # keys: rotary embedding fused into the pass (un-rotated keys read once, rotated rows written once)
+        t = torch.arange(T + 41, device=dev, dtype=torch.float32)
+        inv = 1.0 / (1e6 ** (torch.arange(0, D, 2, device=dev).float() / D))
+        emb = torch.cat([torch.outer(t, inv)] * 2, dim=-1)
+        cos, sin = emb.cos().to(torch.bfloat16), emb.sin().to(torch.bfloat16)
+        k_rot = torch.empty((B, T, Hkv, D), device=dev, dtype=torch.bfloat16)
+        ms_f = _time_fn(torch, lambda: ops.rope_quantize_pack(k_view, cos, sin, 41, k_rot, bits, clip), steps, warmup)
+        ms_r = _time_fn(torch, lambda: ops.rope_rows(k_view, cos, sin, 41, out=k_rot), steps, warmup)
+        ms_q = _time_fn(torch, lambda: ops.quantize_pack(k_rot, bits, clip), steps, warmup)
+        rdf = rd + B * T * Hkv * D * 2      # + the rotated rows written once
+        res["with_rotary_embedding"] = {
+            "fused_us_per_tensor": round(ms_f * 1e3, 1), "algorithmic_bytes": rdf,
+            "achieved_GBps": round(rdf / ms_f / 1e6, 1), "frac_of_hbm_peak": round(rdf / ms_f / 1e6 / HBM_PEAK_GBPS, 4),
+            "two_step_us_per_tensor": round((ms_r + ms_q) * 1e3, 1),
+            "note": "fused: cq_rope_quantize_pack; two-step: cq_rope_rows, then cq_quantize_pack on the rotated tensor"}
+    return res
 
 
 def side_legs(torch, ops, shape, bits, sets, settle_ms=0.0, only_token=False):

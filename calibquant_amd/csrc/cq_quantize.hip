@@ -404,11 +404,27 @@ constexpr int kFRows = 13;                  // rows per thread at most (13 x 256
 constexpr int kFMaxT = kFRows * (kFThreads / 4);
 constexpr int kFGrid = 256;                 // workgroups of the persistent launch (one per compute unit)
 
-template <typename DT, int BITS, int NR>   // NR: rows per thread (T <= NR * 256)
+// Rotary embedding fused into the pass (ROPE): x is the un-rotated key block; every row is rotated as it
+// arrives - rnd(rnd(x * cos) + rotate_half(x) * sin), the arithmetic of the ops the reference runs on the
+// whole key tensor before it quantises the image slice (patch_internvl.py:125-134, 258-260, 295-297) - the
+// rotated row is written out once (the prefill attention and the caller's cache need it) and quantised from
+// the registers.  A channel d pairs with d + 64, so the 32 channels of a slice are then 16 of the lower half
+// and the matching 16 of the upper half (pieces 0, 1 / 2, 3 of a row's four lanes): the partner's raw values
+// are two lanes away, no second read of x.
+struct RopeArgs {
+    const uint16_t* cos;      // (table_rows, 128) in the storage dtype
+    const uint16_t* sin;
+    const int64_t* pos;       // position id of (b, t) at pos[b * pos_sb + t * pos_st]; NULL: pos0 + t
+    int64_t pos_sb, pos_st, pos0, table_rows;
+    uint16_t* out;            // rotated rows, (B, T, H, 128) through element strides
+    int64_t ob, ot, oh;
+};
+
+template <typename DT, int BITS, int NR, bool ROPE = false>   // NR: rows per thread (T <= NR * 256)
 __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* __restrict__ x, QuantGeom g, float clip,
                                                               uint16_t* __restrict__ scale,
                                                               uint16_t* __restrict__ zero,
-                                                              uint8_t* __restrict__ codes) {
+                                                              uint8_t* __restrict__ codes, RopeArgs ra) {
     constexpr int L = (1 << BITS) - 1;
     constexpr float levels = static_cast<float>(L);
     __shared__ __attribute__((aligned(16))) float part_mn[32][kFThreads / 16];   // [channel][wave * 4 + row of 16 lanes]
@@ -430,9 +446,11 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
         const int quarter = (vb >> 3) & 3;
         const uint32_t bh = static_cast<uint32_t>(min(static_cast<int64_t>(vb >> 5) * 8 + (vb & 7), nbh - 1));
         const uint32_t b = g.dH.quot(bh), h = bh - b * g.dH.div;   // B * H < 2^31 on this path
-        return reinterpret_cast<const unsigned char*>(x + static_cast<int64_t>(b) * g.sb + static_cast<int64_t>(h) * g.sh + quarter * 32);
+        return reinterpret_cast<const unsigned char*>(x + static_cast<int64_t>(b) * g.sb + static_cast<int64_t>(h) * g.sh + quarter * (ROPE ? 16 : 32));
     };
-    const uint32_t st_bytes = static_cast<uint32_t>(g.st) * 2u, q_bytes = static_cast<uint32_t>(q4) * 16u;
+    // first channel of the thread's piece, less the slice's own offset (quarter * 32, or quarter * 16 with ROPE)
+    const int chan_t = ROPE ? (q4 >> 1) * 64 + (q4 & 1) * 8 : q4 * 8;
+    const uint32_t st_bytes = static_cast<uint32_t>(g.st) * 2u, q_bytes = static_cast<uint32_t>(chan_t) * 2u;
     auto row_offset = [&](int t) -> uint32_t {   // byte offset of the thread's piece of row min(t, T - 1)
         return static_cast<uint32_t>(__umul24(static_cast<uint32_t>(min(t, g.T - 1)), st_bytes)) + q_bytes;
     };
@@ -452,6 +470,64 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
     const unsigned char* next_base = slice_base(has_next ? vb + gridDim.x : vb);
     int row_i = row;   // opaque per iteration: the row offsets below are recomputed, not kept in registers across the loop
     asm volatile("" : "+v"(row_i));
+    if constexpr (ROPE) {
+        const uint32_t bhc = static_cast<uint32_t>(min(bh, nbh - 1));
+        const uint32_t bb = g.dH.quot(bhc), hh = bhc - bb * g.dH.div;
+        const int chan0 = quarter * 16 + chan_t;
+        uint16_t* orow = ra.out + static_cast<int64_t>(bb) * ra.ob + static_cast<int64_t>(hh) * ra.oh + chan0;
+        const bool upper = (q4 >> 1) != 0;
+        const int64_t* pos_p = ra.pos ? ra.pos + static_cast<int64_t>(bb) * ra.pos_sb : reinterpret_cast<const int64_t*>(ra.cos);
+        const int64_t pos_st = ra.pos ? ra.pos_st : 0;
+        const int64_t trow_max = ra.table_rows - 1;
+        const uint32_t ysign = upper ? 0u : 0x80008000u;   // rotate_half(x) = (-x2, x1): the lower half takes minus its partner
+        // the table rows of GR rows at a time are requested before the first of them is used: every request
+        // is a round trip to the L2, and one row after the other would make a slice wait for NR of them in turn
+        constexpr int GR = 2;
+#pragma unroll
+        for (int i0 = 0; i0 < NR; i0 += GR) {
+            U4 cw[GR], sw[GR];
+#pragma unroll
+            for (int k = 0; k < GR; ++k) {
+                if (i0 + k < NR) {
+                    const int t = min((i0 + k) * (kFThreads / 4) + row_i, g.T - 1);
+                    // no control flow around the loads (the compiler then requests a group's rows side by side):
+                    // without a position tensor the load reads a valid dummy and the select takes pos0 + t
+                    const int64_t pv = pos_p[static_cast<int64_t>(t) * pos_st];
+                    const int64_t pl = ra.pos ? pv : ra.pos0 + t;
+                    // clamped to the table in 32 bits (the host checks table_rows < 2^24)
+                    const uint32_t ps = static_cast<uint32_t>(pl < 0 ? 0 : (pl > trow_max ? trow_max : pl));
+                    cw[k] = *reinterpret_cast<const U4*>(ra.cos + __umul24(ps, 128u) + chan0);
+                    sw[k] = *reinterpret_cast<const U4*>(ra.sin + __umul24(ps, 128u) + chan0);
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < GR; ++k) {
+                if (i0 + k < NR) {
+                    const int i = i0 + k;
+                    const int t = min(i * (kFThreads / 4) + row_i, g.T - 1);
+                    U4 pw;   // the partner's raw piece: the lane two away holds channel d +- 64 of the same row
+#pragma unroll
+                    for (int w = 0; w < 4; ++w)
+                        pw[w] = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(v[i][w]), 0x4E, 0xf, 0xf, true)) ^ ysign;
+                    U4 r4;
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {   // a word (two elements) at a time: few values live at once
+                        const float x0 = Cvt<DT>::lo(v[i][w]), x1 = Cvt<DT>::hi(v[i][w]);
+                        const float y0 = Cvt<DT>::lo(pw[w]), y1 = Cvt<DT>::hi(pw[w]);
+                        const float c0 = Cvt<DT>::lo(cw[k][w]), c1 = Cvt<DT>::hi(cw[k][w]);
+                        const float s0 = Cvt<DT>::lo(sw[k][w]), s1 = Cvt<DT>::hi(sw[k][w]);
+                        const uint32_t o0 = Cvt<DT>::from_float(rnd<DT>(x0 * c0) + y0 * s0);   // y carries the sign of rotate_half
+                        const uint32_t o1 = Cvt<DT>::from_float(rnd<DT>(x1 * c1) + y1 * s1);
+                        r4[w] = o0 | (o1 << 16);
+                    }
+                    v[i] = r4;
+                    // unconditional store: a row past T repeats row T - 1 and a padding slice repeats the last
+                    // (batch, head), so whatever is written twice is written with the same bits
+                    *reinterpret_cast<U4*>(orow + static_cast<int64_t>(t) * ra.ot) = r4;
+                }
+            }
+        }
+    }
     // Both storage types are sign-magnitude, so the extremes of a column follow from three packed
     // 16-bit integer folds of the raw words, two elements per instruction and no unpacking: as
     // signed integers the non-negative values are in value order (the signed maximum is the
@@ -513,7 +589,7 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
             const float diff = rnd<DT>(x_max - x_min);
             const float sc = rnd<DT>(diff * __fdiv_rn(1.0f, levels));
             const float zp = rnd<DT>(__fdiv_rn(-x_min, sc));
-            const int64_t o = bh * g.D + quarter * 32 + c;
+            const int64_t o = bh * g.D + (ROPE ? (c >> 4) * 64 + quarter * 16 + (c & 15) : quarter * 32 + c);
             scale[o] = static_cast<uint16_t>(Cvt<DT>::from_float(sc));
             zero[o] = static_cast<uint16_t>(Cvt<DT>::from_float(zp));
             s_s[c] = sc;
@@ -572,7 +648,8 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
             for (int j = 0; j < 8; ++j)
                 code[j] = ((f[j] >= th[0][j]) ? 1u : 0u) + ((f[j] >= th[1][j]) ? 1u : 0u) + ((f[j] >= th[2][j]) ? 1u : 0u);
         }
-        uint8_t* o = codes + (min(bh, nbh - 1) * g.T + min(t, g.T - 1)) * nb + quarter * (nb / 4);
+        // ROPE: the quad's bytes are two pairs, the lower-half pair at quarter * nb / 8 and the upper-half pair nb / 2 further
+        uint8_t* o = codes + (min(bh, nbh - 1) * g.T + min(t, g.T - 1)) * nb + (ROPE ? quarter * (nb / 8) : quarter * (nb / 4));
         if constexpr (BITS == 1) {
             // The byte is built by eight add-with-carry steps, w = w + w + (f[j] >= th[j]): each
             // comparison leaves its lane mask in a scalar register pair of its own and the add
@@ -608,13 +685,22 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
             w <<= 8 * q4;
             w |= static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(w), 0xB1, 0xf, 0xf, true));
             w |= static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(w), 0x4E, 0xf, 0xf, true));
-            if (q4 == 0 && t < g.T && live) *reinterpret_cast<uint32_t*>(o) = w;
+            if constexpr (ROPE) {
+                if ((q4 & 1) == 0 && t < g.T && live)
+                    *reinterpret_cast<uint16_t*>(o + (q4 >> 1) * (nb / 2)) = static_cast<uint16_t>(w >> (8 * q4));
+            } else {
+                if (q4 == 0 && t < g.T && live) *reinterpret_cast<uint32_t*>(o) = w;
+            }
         } else {
             const uint32_t b0 = (code[0] << 6) | (code[1] << 4) | (code[2] << 2) | code[3];
             const uint32_t b1 = (code[4] << 6) | (code[5] << 4) | (code[6] << 2) | code[7];
             const uint32_t half = b0 | (b1 << 8);
             const uint32_t other = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(half), 0xB1, 0xf, 0xf, true));
-            if ((q4 & 1) == 0 && t < g.T && live) reinterpret_cast<uint32_t*>(o)[q4 >> 1] = half | (other << 16);
+            if constexpr (ROPE) {
+                if ((q4 & 1) == 0 && t < g.T && live) *reinterpret_cast<uint32_t*>(o + (q4 >> 1) * (nb / 2)) = half | (other << 16);
+            } else {
+                if ((q4 & 1) == 0 && t < g.T && live) reinterpret_cast<uint32_t*>(o)[q4 >> 1] = half | (other << 16);
+            }
         }
         // the row is packed: its registers take the same row of the next slice
         if (has_next) v[i] = *reinterpret_cast<const U4*>(next_base + row_offset(t));
@@ -622,23 +708,34 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
     }
 }
 
+// true if the shape goes through the one-pass kernel (x read once, slice by slice in registers)
+static bool one_pass_shape(const QuantGeom& g, const uint8_t* codes) {
+    return g.D == 128 && g.T <= kFMaxT && (reinterpret_cast<uintptr_t>(codes) & 3u) == 0 &&
+           static_cast<int64_t>(g.B) * g.H < (static_cast<int64_t>(1) << 31) && g.st > 0 && g.st * 2 < (1 << 24) &&
+           static_cast<int64_t>(g.T) * g.st * 2 < (static_cast<int64_t>(1) << 31);   // 32-bit row offsets
+}
+
 template <typename DT>
 static int run_quant(const void* x, QuantGeom g, int bits, float clip, uint8_t* codes, void* xq, void* scale,
-                     void* zero, float* ws, hipStream_t st) {
+                     void* zero, float* ws, hipStream_t st, const RopeArgs* rope = nullptr) {
     dim3 grid(g.nchunk, g.H, g.B);
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     uint16_t* sp = static_cast<uint16_t*>(scale);
     uint16_t* zp = static_cast<uint16_t*>(zero);
-    if (!xq && g.D == 128 && g.T <= kFMaxT && (reinterpret_cast<uintptr_t>(codes) & 3u) == 0 &&
-        static_cast<int64_t>(g.B) * g.H < (static_cast<int64_t>(1) << 31) &&
-        g.st > 0 && g.st * 2 < (1 << 24) && static_cast<int64_t>(g.T) * g.st * 2 < (static_cast<int64_t>(1) << 31)) {   // 32-bit row offsets
+    if (rope && (xq || !one_pass_shape(g, codes))) return CQ_ERR_UNSUPPORTED;
+    if (!xq && one_pass_shape(g, codes)) {
         // x fits a workgroup's registers slice by slice: one pass
         const int64_t bh8 = (static_cast<int64_t>(g.B) * g.H + 7) / 8;
         // persistent: at most one workgroup per compute unit and a multiple of 32 of them
         const int64_t nsl = bh8 * 32;
         const dim3 fgrid(static_cast<unsigned>(nsl < kFGrid ? nsl : kFGrid));
         const int nr = (g.T + kFThreads / 4 - 1) / (kFThreads / 4);
-#define CQ_FUSED(B_, N_) hipLaunchKernelGGL((fused_pack_kernel<DT, B_, N_>), fgrid, dim3(kFThreads), 0, st, xp, g, clip, sp, zp, codes)
+        const RopeArgs ra = rope ? *rope : RopeArgs{};
+#define CQ_FUSED(B_, N_)                                                                                              \
+        do {                                                                                                          \
+            if (rope) hipLaunchKernelGGL((fused_pack_kernel<DT, B_, N_, true>), fgrid, dim3(kFThreads), 0, st, xp, g, clip, sp, zp, codes, ra);  \
+            else hipLaunchKernelGGL((fused_pack_kernel<DT, B_, N_, false>), fgrid, dim3(kFThreads), 0, st, xp, g, clip, sp, zp, codes, ra);      \
+        } while (0)
         if (bits == 1) {
             if (nr <= 4) CQ_FUSED(1, 4); else if (nr <= 8) CQ_FUSED(1, 8); else CQ_FUSED(1, 13);
         } else {
@@ -698,7 +795,7 @@ static int run_quant_tensor(const void* x, QuantGeom g, int bits, float clip, vo
 
 static int quant_entry(const void* x, int dtype, int B, int T, int H, int D, int64_t sb, int64_t st, int64_t sh,
                        int bits, float clip, uint8_t* codes, void* xq, void* scale, void* zero, void* ws,
-                       size_t ws_bytes, cq_stream_t stream) {
+                       size_t ws_bytes, cq_stream_t stream, const RopeArgs* rope = nullptr) {
     if (!x || !scale || !zero || (!codes && !xq)) return CQ_ERR_NULL;
     if (dtype != CQ_BF16 && dtype != CQ_FP16) return CQ_ERR_DTYPE;
     if (bits != 1 && bits != 2) return CQ_ERR_UNSUPPORTED;
@@ -718,8 +815,54 @@ static int quant_entry(const void* x, int dtype, int B, int T, int H, int D, int
     g.dH.set(static_cast<uint32_t>(H));
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == CQ_BF16)
-        return run_quant<BF16>(x, g, bits, clip, codes, xq, scale, zero, static_cast<float*>(ws), s);
-    return run_quant<FP16>(x, g, bits, clip, codes, xq, scale, zero, static_cast<float*>(ws), s);
+        return run_quant<BF16>(x, g, bits, clip, codes, xq, scale, zero, static_cast<float*>(ws), s, rope);
+    return run_quant<FP16>(x, g, bits, clip, codes, xq, scale, zero, static_cast<float*>(ws), s, rope);
+}
+
+// Rotary embedding of the rows of a (B, T, H, 128) view, the same arithmetic as above: one thread per
+// (row, head, 8 channels of the lower half and the matching 8 of the upper half).
+template <typename DT>
+__global__ __launch_bounds__(256) void rope_rows_kernel(const uint16_t* __restrict__ x, QuantGeom g, RopeArgs ra) {
+    typedef uint32_t U4 __attribute__((ext_vector_type(4)));
+    const int64_t gid = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    const int64_t total = static_cast<int64_t>(g.B) * g.T * g.H * 8;
+    if (gid >= total) return;
+    const int p8 = static_cast<int>(gid & 7);
+    int64_t r = gid >> 3;
+    const int h = static_cast<int>(r % g.H); r /= g.H;
+    const int t = static_cast<int>(r % g.T);
+    const int b = static_cast<int>(r / g.T);
+    const uint16_t* xr = x + b * g.sb + static_cast<int64_t>(t) * g.st + static_cast<int64_t>(h) * g.sh + p8 * 8;
+    int64_t ps = ra.pos ? ra.pos[b * ra.pos_sb + static_cast<int64_t>(t) * ra.pos_st] : ra.pos0 + t;
+    ps = ps < 0 ? 0 : (ps >= ra.table_rows ? ra.table_rows - 1 : ps);
+    const U4 lo = *reinterpret_cast<const U4*>(xr), hi = *reinterpret_cast<const U4*>(xr + 64);
+    const U4 cl = *reinterpret_cast<const U4*>(ra.cos + ps * 128 + p8 * 8), ch = *reinterpret_cast<const U4*>(ra.cos + ps * 128 + 64 + p8 * 8);
+    const U4 sl = *reinterpret_cast<const U4*>(ra.sin + ps * 128 + p8 * 8), sh = *reinterpret_cast<const U4*>(ra.sin + ps * 128 + 64 + p8 * 8);
+    float x1[8], x2[8], c1[8], c2[8], s1[8], s2[8];
+    unpack8<DT>(lo, x1); unpack8<DT>(hi, x2); unpack8<DT>(cl, c1); unpack8<DT>(ch, c2); unpack8<DT>(sl, s1); unpack8<DT>(sh, s2);
+    uint32_t o1[8], o2[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        o1[j] = Cvt<DT>::from_float(rnd<DT>(x1[j] * c1[j]) + (-x2[j]) * s1[j]);
+        o2[j] = Cvt<DT>::from_float(rnd<DT>(x2[j] * c2[j]) + x1[j] * s2[j]);
+    }
+    U4 r1, r2;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) { r1[w] = o1[2 * w] | (o1[2 * w + 1] << 16); r2[w] = o2[2 * w] | (o2[2 * w + 1] << 16); }
+    uint16_t* orow = ra.out + b * ra.ob + static_cast<int64_t>(t) * ra.ot + static_cast<int64_t>(h) * ra.oh + p8 * 8;
+    *reinterpret_cast<U4*>(orow) = r1;
+    *reinterpret_cast<U4*>(orow + 64) = r2;
+}
+
+static int check_rope(const void* cos_table, const void* sin_table, int64_t table_rows, const int64_t* pos,
+                      void* out, int64_t ob, int64_t ot, int64_t oh, int D) {
+    if (!cos_table || !sin_table || !out) return CQ_ERR_NULL;
+    if (D != 128) return CQ_ERR_UNSUPPORTED;
+    if (table_rows < 1 || table_rows >= (1 << 24)) return CQ_ERR_SHAPE;
+    if (!aligned16(cos_table) || !aligned16(sin_table) || !aligned16(out) || (ob % 8) || (ot % 8) || (oh % 8) ||
+        (pos && (reinterpret_cast<uintptr_t>(pos) & 7u)))
+        return CQ_ERR_ALIGN;
+    return CQ_OK;
 }
 
 // ---- per-token value quantiser --------------------------------------------------------
@@ -872,6 +1015,50 @@ int cq_quantize_pack(const void* x, int dtype, int B, int T, int H, int D, int64
     if (!codes) return CQ_ERR_NULL;
     return cq::quant_entry(x, dtype, B, T, H, D, stride_b, stride_t, stride_h, bits, clip, codes, nullptr, scale,
                            zero, workspace, workspace_bytes, stream);
+}
+
+int cq_rope_quantize_pack(const void* x, int dtype, int B, int T, int H, int D, int64_t stride_b, int64_t stride_t,
+                          int64_t stride_h, const void* cos_table, const void* sin_table, int64_t table_rows,
+                          const int64_t* pos, int64_t pos_stride_b, int64_t pos_stride_t, int64_t pos0,
+                          void* x_rot, int64_t rot_stride_b, int64_t rot_stride_t, int64_t rot_stride_h,
+                          int bits, float clip, uint8_t* codes, void* scale, void* zero,
+                          void* workspace, size_t workspace_bytes, cq_stream_t stream) {
+    if (!codes) return CQ_ERR_NULL;
+    int rc = cq::check_rope(cos_table, sin_table, table_rows, pos, x_rot, rot_stride_b, rot_stride_t, rot_stride_h, D);
+    if (rc != CQ_OK) return rc;
+    cq::RopeArgs ra;
+    ra.cos = static_cast<const uint16_t*>(cos_table); ra.sin = static_cast<const uint16_t*>(sin_table);
+    ra.pos = pos; ra.pos_sb = pos_stride_b; ra.pos_st = pos_stride_t; ra.pos0 = pos0; ra.table_rows = table_rows;
+    ra.out = static_cast<uint16_t*>(x_rot); ra.ob = rot_stride_b; ra.ot = rot_stride_t; ra.oh = rot_stride_h;
+    return cq::quant_entry(x, dtype, B, T, H, D, stride_b, stride_t, stride_h, bits, clip, codes, nullptr, scale,
+                           zero, workspace, workspace_bytes, stream, &ra);
+}
+
+int cq_rope_rows(const void* x, int dtype, int B, int T, int H, int D, int64_t stride_b, int64_t stride_t,
+                 int64_t stride_h, const void* cos_table, const void* sin_table, int64_t table_rows,
+                 const int64_t* pos, int64_t pos_stride_b, int64_t pos_stride_t, int64_t pos0,
+                 void* x_rot, int64_t rot_stride_b, int64_t rot_stride_t, int64_t rot_stride_h, cq_stream_t stream) {
+    if (!x) return CQ_ERR_NULL;
+    if (dtype != CQ_BF16 && dtype != CQ_FP16) return CQ_ERR_DTYPE;
+    if (B < 1 || T < 1 || H < 1) return CQ_ERR_SHAPE;
+    int rc = cq::check_rope(cos_table, sin_table, table_rows, pos, x_rot, rot_stride_b, rot_stride_t, rot_stride_h, D);
+    if (rc != CQ_OK) return rc;
+    if ((stride_b % 8) || (stride_t % 8) || (stride_h % 8) || !cq::aligned16(x)) return CQ_ERR_ALIGN;
+    cq::QuantGeom g = {};
+    g.B = B; g.T = T; g.H = H; g.D = D; g.sb = stride_b; g.st = stride_t; g.sh = stride_h;
+    cq::RopeArgs ra;
+    ra.cos = static_cast<const uint16_t*>(cos_table); ra.sin = static_cast<const uint16_t*>(sin_table);
+    ra.pos = pos; ra.pos_sb = pos_stride_b; ra.pos_st = pos_stride_t; ra.pos0 = pos0; ra.table_rows = table_rows;
+    ra.out = static_cast<uint16_t*>(x_rot); ra.ob = rot_stride_b; ra.ot = rot_stride_t; ra.oh = rot_stride_h;
+    const int64_t total = static_cast<int64_t>(B) * T * H * 8;
+    const int64_t blocks = (total + 255) / 256;
+    if (blocks > 0x7fffffff) return CQ_ERR_SHAPE;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint16_t* xp = static_cast<const uint16_t*>(x);
+    if (dtype == CQ_BF16) hipLaunchKernelGGL(cq::rope_rows_kernel<cq::BF16>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st, xp, g, ra);
+    else hipLaunchKernelGGL(cq::rope_rows_kernel<cq::FP16>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st, xp, g, ra);
+    CQ_LAUNCH_CHECK();
+    return CQ_OK;
 }
 
 int cq_quantize_pack_token(const void* x, int dtype, int B, int T, int H, int D, int64_t stride_b, int64_t stride_t,

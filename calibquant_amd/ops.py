@@ -62,6 +62,75 @@ def quantize_pack(x: torch.Tensor, bits: int, clip: float) -> Tuple[torch.Tensor
     return codes, scale, zero
 
 
+def _rope_args(x, cos, sin, pos, out):
+    """Common argument block of the two rotary entry points."""
+    for t, n in ((cos, "cos"), (sin, "sin"), (out, "out")):
+        _need_gpu(t, n)
+        if t.dtype != x.dtype:
+            raise _lib.CalibQuantError("rope: cos, sin and out must share x's dtype")
+    if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != x.shape[3] or not (cos.is_contiguous() and sin.is_contiguous()):
+        raise _lib.CalibQuantError("rope: cos / sin must be contiguous (rows, D) tables")
+    if out.shape != x.shape or out.stride(3) != 1:
+        raise _lib.CalibQuantError("rope: out must be shaped like x with a contiguous last axis")
+    B, T = x.shape[0], x.shape[1]
+    if isinstance(pos, int):
+        pos_args = (None, 0, 0, int(pos))
+        keep = None
+    else:
+        _need_gpu(pos, "pos")
+        if pos.dtype != torch.int64 or pos.shape != (B, T):
+            raise _lib.CalibQuantError("rope: pos must be an int64 (B, T) tensor or an int (first position of an arange)")
+        pos_args = (pos.data_ptr(), pos.stride(0), pos.stride(1), 0)
+        keep = pos
+    return (x.data_ptr(), _storage_dtype(x, "x"), *x.shape, x.stride(0), x.stride(1), x.stride(2),
+            cos.data_ptr(), sin.data_ptr(), cos.shape[0], *pos_args,
+            out.data_ptr(), out.stride(0), out.stride(1), out.stride(2)), keep
+
+
+def rope_rows(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, pos, out: Optional[torch.Tensor] = None):
+    """Rotary embedding of x (B, T, H, D) (any b/t/h strides) with the reference's rounding:
+    rnd(rnd(x*cos) + rotate_half(x)*sin).  cos / sin: (rows, D) tables; pos: int64 (B, T) position
+    ids (any strides) or an int p0 for positions p0 + t.  Writes `out` (shaped like x) or a new
+    contiguous tensor."""
+    _need_gpu(x, "x")
+    if x.dim() != 4 or x.stride(3) != 1:
+        raise _lib.CalibQuantError("x must be (B, T, H, D) with a contiguous last axis")
+    if out is None:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    args, keep = _rope_args(x, cos, sin, pos, out)
+    with torch.cuda.device(x.device):
+        rc = _lib.load().cq_rope_rows(*args, _stream(x))
+    _lib.check(rc, "cq_rope_rows")
+    return out
+
+
+def rope_quantize_pack(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, pos, out: torch.Tensor,
+                       bits: int, clip: float):
+    """`quantize_pack(rope(x))` in one pass over x: x (B, T, H, D) is the UN-rotated key block; the
+    rotated rows are written to `out` (shaped like x) and quantised from the registers.  Returns
+    codes uint8 (B, H, T, D*bits/8), scale (B, H, D), zero (B, H, D), bit-identical to
+    `quantize_pack(rope_rows(x, ...), bits, clip)`.  Raises `CalibQuantError` (unsupported) for shapes
+    outside the one-pass path (T > 3 328 or D != 128)."""
+    _need_gpu(x, "x")
+    if x.dim() != 4 or x.stride(3) != 1:
+        raise _lib.CalibQuantError("x must be (B, T, H, D) with a contiguous last axis")
+    B, T, H, D = x.shape
+    args, keep = _rope_args(x, cos, sin, pos, out)
+    lib = _lib.load()
+    codes = torch.empty((B, H, T, D * bits // 8), dtype=torch.uint8, device=x.device)
+    scale = torch.empty((B, H, D), dtype=x.dtype, device=x.device)
+    zero = torch.empty((B, H, D), dtype=x.dtype, device=x.device)
+    ws = _workspace(lib.cq_quantize_pack_workspace(B, T, H, D), x.device)
+    with torch.cuda.device(x.device):
+        rc = lib.cq_rope_quantize_pack(*args, int(bits), float(clip), codes.data_ptr(), scale.data_ptr(),
+                                       zero.data_ptr(), ws.data_ptr(), ws.numel(), _stream(x))
+    _lib.check(rc, "cq_rope_quantize_pack")
+    return codes, scale, zero
+
+
+ROPE_FUSED_MAX_T = 3328      # the one-pass quantiser holds a (batch, head) slice of at most this many rows
+
+
 def quantize_pack_token(x: torch.Tensor, bits: int, group_size: int = 32):
     """Per-token min-max quantiser of the values (`v_mode = token`): x (B, T, H, D) view, bf16 or
     fp16, D = 128, groups of 32 channels.  Returns words int32 (B, H, T, D*bits/32) (first channel

@@ -165,15 +165,33 @@ def forward_internlm2_calibquant(self, hidden_states: torch.Tensor, attention_ma
             and position_ids.dtype == torch.int64 and position_ids.numel() == bsz and qkv.is_contiguous()
             and qkv.dtype in (torch.bfloat16, torch.float16)):
         return _decode_step_fused(self, qkv, position_ids, past_key_value, attention_mask, use_cache)
-    query_states = qkv[..., :G, :].reshape(bsz, q_len, Hq, D).transpose(1, 2)     # (B, Hq, q, D)
-    key_states = qkv[..., -2, :].transpose(1, 2)                                   # (B, Hkv, q, D)
-    value_states = qkv[..., -1, :].transpose(1, 2)
-
+    value_states = qkv[..., -1, :].transpose(1, 2)                                 # (B, Hkv, q, D)
     kv_seq_len = q_len
     if past_key_value is not None:
         kv_seq_len += past_key_value[0].shape[-2] + T                               # patch_internvl.py:246-251
     cos, sin = self.rotary_emb(value_states, seq_len=kv_seq_len)
-    query_states, key_states = apply_rotary_pos_emb(query_states, key_states, cos, sin, position_ids)
+    # Prefill on the GPU: the rotary embedding runs in HIP kernels with the rounding of the reference's op
+    # chain - queries and the keys outside the image block in `cq_rope_rows`, the image block of the keys
+    # inside the quantise-and-pack pass itself (`cq_rope_quantize_pack`: the un-rotated keys are read once,
+    # the rotated rows written once and quantised from the registers).  The reference rotates the whole
+    # tensors with a chain of torch ops first (patch_internvl.py:258-260) and quantises afterwards (:295-297).
+    hip_rope = (q_len > 1 and qkv.is_cuda and qkv.dtype in (torch.bfloat16, torch.float16) and D == 128
+                and position_ids is not None and position_ids.is_cuda and position_ids.dtype == torch.int64
+                and tuple(position_ids.shape) == (bsz, q_len))
+    k_rot = None
+    if hip_rope:
+        cos, sin = cos.contiguous(), sin.contiguous()
+        q_rot = torch.empty((bsz, q_len, Hkv, G, D), dtype=qkv.dtype, device=qkv.device)
+        for gq in range(G):     # one launch per query head of a group: each is a (B, q, Hkv, D) view of the projection
+            ops.rope_rows(qkv[..., gq, :], cos, sin, position_ids, out=q_rot[..., gq, :])
+        query_states = q_rot.view(bsz, q_len, Hq, D).transpose(1, 2)               # (B, Hq, q, D)
+        k_raw = qkv[..., -2, :]                                                    # (B, q, Hkv, D), un-rotated
+        k_rot = torch.empty((bsz, q_len, Hkv, D), dtype=qkv.dtype, device=qkv.device)
+        key_states = k_rot.transpose(1, 2)                                         # filled in the prefill branch
+    else:
+        query_states = qkv[..., :G, :].reshape(bsz, q_len, Hq, D).transpose(1, 2)  # (B, Hq, q, D)
+        key_states = qkv[..., -2, :].transpose(1, 2)                               # (B, Hkv, q, D)
+        query_states, key_states = apply_rotary_pos_emb(query_states, key_states, cos, sin, position_ids)
 
     if not hasattr(self, "_cq_window"):
         self._cq_window = GrowingKV()
@@ -186,10 +204,22 @@ def forward_internlm2_calibquant(self, hidden_states: torch.Tensor, attention_ma
         if S + T > q_len:
             raise CalibQuantError(f"prompt of {q_len} tokens is shorter than sprompt_len + image tokens = {S + T}")
         self._cq_call = None
+        fused_rope = hip_rope and 0 < T <= ops.ROPE_FUSED_MAX_T
+        if hip_rope:
+            if fused_rope:      # image block: rotated inside the quantiser; the rows around it on their own
+                ck, ks, kz = ops.rope_quantize_pack(k_raw[:, S:S + T], cos, sin, position_ids[:, S:S + T],
+                                                    k_rot[:, S:S + T], self.bits_k, self.scale_k)
+                if S > 0:
+                    ops.rope_rows(k_raw[:, :S], cos, sin, position_ids[:, :S], out=k_rot[:, :S])
+                if S + T < q_len:
+                    ops.rope_rows(k_raw[:, S + T:], cos, sin, position_ids[:, S + T:], out=k_rot[:, S + T:])
+            else:               # no image block, or one beyond the one-pass quantiser: rotate everything first
+                ops.rope_rows(k_raw, cos, sin, position_ids, out=k_rot)
         if T > 0:
             k_img = key_states[:, :, S:S + T, :].transpose(1, 2)      # (B, T, Hkv, D) strided views
             v_img = value_states[:, :, S:S + T, :].transpose(1, 2)
-            ck, ks, kz = ops.quantize_pack(k_img, self.bits_k, self.scale_k)
+            if not fused_rope:
+                ck, ks, kz = ops.quantize_pack(k_img, self.bits_k, self.scale_k)
             if self.v_mode == "token":
                 cv, vs, vz = ops.quantize_pack_token(v_img, self.bits_v)      # words, scale, minimum per (token, group)
             else:

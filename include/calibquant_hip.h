@@ -68,6 +68,45 @@ int cq_quantize_pack(const void* x, int dtype, int B, int T, int H, int D,
                      void* workspace, size_t workspace_bytes, cq_stream_t stream);
 
 /* ------------------------------------------------------------------------
+ * Prefill, keys: rotary embedding fused into the quantise-and-pack pass.
+ * Replaces, for the image slice of the key tensor, the rotary embedding of
+ * the whole key tensor (patch_internvl.py:258-260 with :119-138) followed by
+ * cq_quantize_pack's chain (:295-297, 325-339): x is the UN-rotated key
+ * block (B, T, H, 128) of the fused projection output; every row is rotated
+ * as it arrives, rnd(rnd(x*cos) + rotate_half(x)*sin) with the product added
+ * in fp32 (the arithmetic of `copy_().mul_()` + `addcmul_`, :125-128), the
+ * rotated row is written once to x_rot (the prefill attention and the cache
+ * of the remaining tokens need it) and quantised from the registers: the keys
+ * are read from HBM once and nothing is read back.
+ * cos_table, sin_table: (table_rows, 128), storage dtype, 16-byte aligned.
+ * pos: device int64, position id of (b, t) at pos[b*pos_stride_b +
+ * t*pos_stride_t] (clamped to the table), or NULL for positions pos0 + t.
+ * x_rot: (B, T, H, 128) through element strides (multiples of 8).
+ * codes / scale / zero / workspace as for cq_quantize_pack; the results are
+ * bit-identical to cq_quantize_pack on the rotated tensor.
+ * Shapes outside the one-pass path (T > 3 328, D != 128) return
+ * CQ_ERR_UNSUPPORTED: rotate with cq_rope_rows, then cq_quantize_pack. */
+int cq_rope_quantize_pack(const void* x, int dtype, int B, int T, int H, int D,
+                          int64_t stride_b, int64_t stride_t, int64_t stride_h,
+                          const void* cos_table, const void* sin_table, int64_t table_rows,
+                          const int64_t* pos, int64_t pos_stride_b, int64_t pos_stride_t, int64_t pos0,
+                          void* x_rot, int64_t rot_stride_b, int64_t rot_stride_t, int64_t rot_stride_h,
+                          int bits, float clip, uint8_t* codes, void* scale, void* zero,
+                          void* workspace, size_t workspace_bytes, cq_stream_t stream);
+
+/* The rotary embedding alone, same arithmetic, for the rows that are not
+ * quantised (queries; system-prompt and text keys): x (B, T, H, 128) through
+ * strides -> x_rot (B, T, H, 128) through strides; one launch instead of the
+ * reference's chain of torch ops over the whole tensor
+ * (patch_internvl.py:119-138). */
+int cq_rope_rows(const void* x, int dtype, int B, int T, int H, int D,
+                 int64_t stride_b, int64_t stride_t, int64_t stride_h,
+                 const void* cos_table, const void* sin_table, int64_t table_rows,
+                 const int64_t* pos, int64_t pos_stride_b, int64_t pos_stride_t, int64_t pos0,
+                 void* x_rot, int64_t rot_stride_b, int64_t rot_stride_t, int64_t rot_stride_h,
+                 cq_stream_t stream);
+
+/* ------------------------------------------------------------------------
  * Per-token value quantiser: the reference's
  * triton_quantize_and_pack_along_last_dim(data, group_size, bit)
  * (qjl/new_pack.py:53-82), the source of the `v_mode = token` layout that
