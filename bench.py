@@ -367,7 +367,7 @@ def model_leg(torch, batch=64, tiles=13, sys_len=41, text_len=23, new_tokens=128
 
     def drop_state():
         for layer in model.language_model.model.layers:      # drop the KV state before the next run
-            for name in ("_kv", "_cq_window", "_cq_call", "_cq_stats", "encoded_features_k", "encoded_features_v"):
+            for name in ("_kv", "_cq_window", "_cq_call", "_cq_step", "_cq_stats", "encoded_features_k", "encoded_features_v"):
                 if hasattr(layer.attention, name):
                     delattr(layer.attention, name)
         torch.cuda.empty_cache()

@@ -109,6 +109,30 @@ def load() -> C.CDLL:
     return lib
 
 
+SHIM_PATH = os.path.join(_HERE, "lib", "_cq_torch_step.so")
+_shim = None
+
+
+def load_step_shim():
+    """The host shim `_cq_torch_step` (C++ over torch's headers; `LayerStep` runs the steady-state decode
+    step of one attention layer in one call).  Built by `python -m calibquant_amd.build`; raises if missing."""
+    global _shim
+    if _shim is None:
+        if not os.path.exists(SHIM_PATH):
+            raise CalibQuantError(f"{SHIM_PATH} is missing: build it with `python -m calibquant_amd.build`")
+        import importlib.util
+
+        import torch  # noqa: F401  (the shim links torch's libraries; they must be loaded first)
+        load()
+        spec = importlib.util.spec_from_file_location("_cq_torch_step", SHIM_PATH)
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        if mod.library_version() != load().cq_version():
+            raise CalibQuantError("the host shim and the HIP library were built from different sources")
+        _shim = mod
+    return _shim
+
+
 def check(status: int, what: str) -> None:
     if status != 0:
         lib = load()

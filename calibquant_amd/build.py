@@ -2,6 +2,8 @@
 
 Run `python -m calibquant_amd.build`.  hipcc cross-compiles for gfx950 without
 a GPU.  The built library is git-ignored and is loaded by `calibquant_amd._lib`.
+The second product is the host shim `_cq_torch_step.so` (C++ over torch's headers,
+host compiler), which the eager decode step of the attention patch calls.
 """
 from __future__ import annotations
 
@@ -52,6 +54,34 @@ def build(verbose: bool = True, jobs: int = 4) -> str:
     return LIBPATH
 
 
+SHIM_SRC = os.path.join(CSRC, "cq_torch_step.cpp")
+SHIM_NAME = "_cq_torch_step"
+SHIMPATH = os.path.join(LIBDIR, SHIM_NAME + ".so")
+
+
+def build_torch_shim(verbose: bool = True) -> str:
+    """The host shim between PyTorch and the C-ABI library (`calibquant_amd/lib/_cq_torch_step.so`): plain
+    C++ over torch's headers, no kernels, so the host compiler builds it; it links the HIP library beside
+    it (run-path $ORIGIN) and the torch libraries of the interpreter that builds it."""
+    import sysconfig
+
+    import torch
+    tdir = os.path.dirname(torch.__file__)
+    cxx = os.environ.get("CXX", "g++")
+    cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unknown-pragmas",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_API_INCLUDE_EXTENSION_H",
+           "-DTORCH_EXTENSION_NAME=" + SHIM_NAME, "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI),
+           "-I" + os.path.join(tdir, "include"), "-I" + os.path.join(tdir, "include", "torch", "csrc", "api", "include"),
+           "-I/opt/rocm/include", "-I" + sysconfig.get_paths()["include"], "-I" + os.path.join(ROOT, "include"),
+           SHIM_SRC, "-o", SHIMPATH,
+           "-L" + os.path.join(tdir, "lib"), "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch",
+           "-ltorch_python", "-L" + LIBDIR, "-lcalibquant_hip", "-Wl,-rpath,$ORIGIN"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    return SHIMPATH
+
+
 def _drain(procs):
     while procs:
         src, p = procs.pop(0)
@@ -66,4 +96,5 @@ def _drain(procs):
 
 if __name__ == "__main__":
     print(build())
+    print(build_torch_shim())
     sys.exit(0)

@@ -15,13 +15,14 @@ and is not provided.
 """
 from __future__ import annotations
 
+import ctypes as C
 import os
 import warnings
 from typing import Optional, Tuple
 
 import torch
 
-from . import ops
+from . import _lib, ops
 from ._lib import CalibQuantError
 from .kvbuffer import GrowingKV
 
@@ -137,6 +138,16 @@ def forward_internlm2_calibquant(self, hidden_states: torch.Tensor, attention_ma
     (K, V) of shape (B, Hkv, R, D) holding the system prompt rows [0, S), the text rows and every
     generated token; the image rows live packed on the module
     (`encoded_features_k/v`, `scale_key/value`, `zero_point_key/value`, `unique_values_k/v`)."""
+    # steady-state decode: the step object the first decode step prepared runs the whole step (rotary
+    # embedding + window append launch, attention launch) in one call into the host shim; it declines
+    # (returns None) when this is not the next token of the window it owns
+    fast = self.__dict__.get("_cq_step")
+    if (fast is not None and attention_mask is None and past_key_value is not None and position_ids is not None
+            and not kwargs and hidden_states.shape[1] == 1):
+        got = fast[0].step(self.wqkv(hidden_states), position_ids, past_key_value[0])
+        if got is not None:
+            return self.wo(got[0]), None, ((got[1], got[2]) if use_cache else None)
+        del self.__dict__["_cq_step"]
     # hyper-parameters published on the module, as patch_internvl.py:175-191 does
     self.sprompt_len = getattr(self, "cq_sprompt_len", SPROMPT_LEN)
     self.bits_k = self.bits_v = getattr(self, "cq_bits", BITS_KV)
@@ -204,6 +215,7 @@ def forward_internlm2_calibquant(self, hidden_states: torch.Tensor, attention_ma
         if S + T > q_len:
             raise CalibQuantError(f"prompt of {q_len} tokens is shorter than sprompt_len + image tokens = {S + T}")
         self._cq_call = None
+        self.__dict__.pop("_cq_step", None)
         fused_rope = hip_rope and 0 < T <= ops.ROPE_FUSED_MAX_T
         if hip_rope:
             if fused_rope:      # image block: rotated inside the quantiser; the rows around it on their own
@@ -346,6 +358,14 @@ def _decode_step_fused(self, qkv, position_ids, past_key_value, attention_mask, 
                              f"but is {attention_mask.size()}")
         mask = attention_mask[:, 0, 0, :]
     out = _attend(self, q1, k_res, v_res, mask)
+    call = getattr(self, "_cq_call", None)
+    if (mask is None and use_cache and call is not None and call.workspace_bytes == 0 and call.args.B == bsz
+            and not getattr(self, "cq_no_step_shim", False)):
+        # from the next token on the host shim runs this whole function in one call; it takes over the
+        # window buffers (this step's past_key_value are views of them) and keeps `call`'s tensors alive
+        shim = _lib.load_step_shim()
+        self.__dict__["_cq_step"] = (shim.LayerStep(C.addressof(call.args), C.sizeof(call.args), tabs[0], tabs[1],
+                                                    win.k, win.v, win.len, rows), call)
     return self.wo(out.reshape(bsz, 1, self.hidden_size)), None, past_key_value
 
 

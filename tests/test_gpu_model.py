@@ -67,18 +67,20 @@ def test_patched_forward_decode_matches_oracle_on_one_layer():
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_fused_decode_step_equals_the_unfused_op_chain(dtype):
-    """Several decode steps through the one-launch split + rotary + append path and through the
-    chain of torch ops (forced by int32 position ids): same outputs and same window, bit for bit."""
+    """Several decode steps through the one-launch split + rotary + append path - once driven by the host
+    shim's `LayerStep` (the default), once by the Python call objects - and through the chain of torch ops
+    (forced by int32 position ids): same outputs and same window, bit for bit."""
     from calibquant_amd import patch_internvl as pi
     from calibquant_amd.internlm2 import InternLM2Attention, InternLM2Config
     cfg = InternLM2Config.tiny()
     B, S, T, TXT = 3, 4, 130, 9
     N = S + T + TXT
     outs, wins = [], []
-    for fused in (True, False):
+    for fused, shim in ((True, True), (True, False), (False, False)):
         torch.manual_seed(7)
         att = InternLM2Attention(cfg).cuda().to(dtype)
         att.cq_sprompt_len, att.cq_image_token_num = S, T
+        att.cq_no_step_shim = not shim
         x = torch.randn(B, N, cfg.hidden_size, device="cuda", dtype=dtype)
         pos = torch.arange(N, device="cuda")[None].expand(B, N)
         with torch.no_grad():
@@ -92,11 +94,17 @@ def test_fused_decode_step_equals_the_unfused_op_chain(dtype):
                 if i % 37 == 0 or i == 299:
                     step_out.append(o.clone())
         assert hasattr(att, "_cq_rope_call") == fused
+        if shim:    # every step after the first went through the shim, which regrew the window on the way
+            step = att._cq_step[0]
+            assert step.steps == 299 and step.length == S + TXT + 300 and step.capacity >= step.length
+        else:
+            assert "_cq_step" not in att.__dict__
         outs.append(torch.stack(step_out))
         wins.append((past[0].clone(), past[1].clone()))
     assert wins[0][0].shape == (B, cfg.num_key_value_heads, S + TXT + 300, 128)
-    assert torch.equal(wins[0][0], wins[1][0]) and torch.equal(wins[0][1], wins[1][1])
-    assert torch.equal(outs[0], outs[1])
+    for other in (1, 2):
+        assert torch.equal(wins[0][0], wins[other][0]) and torch.equal(wins[0][1], wins[other][1])
+        assert torch.equal(outs[0], outs[other])
 
 
 def test_patched_model_without_image_tokens_equals_the_fp_model():
@@ -154,7 +162,7 @@ def test_patch_model_and_custom_generate_end_to_end(tower):
         assert os.environ["IMAGE_TOKEN_NUM"] == str(T)
         att = m.language_model.model.layers[0].attention
         assert att.encoded_features_k.shape == (B, 2, T, 16) and att.encoded_features_k.dtype == torch.uint8
-        assert att._cq_window.len == S + txt + 7
+        assert att._cq_step[0].length == S + txt + 7
         out2 = m.generate(pixel_values=pix, input_ids=ids, max_new_tokens=8)
         assert torch.equal(out, out2)
     finally:

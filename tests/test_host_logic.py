@@ -219,3 +219,17 @@ def test_image_token_count_is_reread_from_the_environment_every_forward(monkeypa
     assert pi._image_token_num(att) == 512
     att.cq_image_token_num = 256                            # the explicit channel (custom_generate sets it)
     assert pi._image_token_num(att) == 256
+
+
+def test_host_shim_loads_and_matches_the_library():
+    """`_cq_torch_step.so` (the C++ step object of the eager decode path) imports, exposes `LayerStep`
+    and was built against the same library version; no GPU call is made."""
+    from calibquant_amd import _lib
+    shim = _lib.load_step_shim()
+    assert shim.library_version() == _lib.load().cq_version()
+    assert {"step", "length", "steps", "capacity"} <= set(dir(shim.LayerStep))
+    import ctypes as C
+    import torch
+    with pytest.raises(Exception):      # CPU tensors / wrong block size are refused before any launch
+        shim.LayerStep(C.addressof(_lib.DecodeArgs()), 8, torch.zeros(1), torch.zeros(1), torch.zeros(1),
+                       torch.zeros(1), 0, torch.zeros(1, dtype=torch.int64))
