@@ -27,9 +27,12 @@
 //            the same workgroup (packed dot2 for q.K) and are merged at the end.
 //
 // When the chunk does not cover all T tokens (long context or small batch)
-// a first launch publishes the per-chunk logit min / max, the main launch
-// recomputes its chunk's logits against the global min / max and writes an
-// (m, l, acc) partial, and a merge launch combines the partials.
+// a first launch computes every chunk's logits and publishes the per-chunk min / max;
+// the main launch recomputes its chunk's logits (or, where the packed K row is more
+// bytes than the logits - 2 bits, or fewer than four heads per unit - reads back what
+// the first launch left in a buffer, fp32, instead of building the table and doing the
+// look-ups again), exponentiates against the global min / max and writes an (m, l, acc)
+// partial; the last workgroup of a unit to get there combines the unit's partials.
 //
 // Everything here is HBM / LDS / VALU work; no matrix-core instructions.
 #include "cq_common.h"
@@ -65,6 +68,10 @@ struct DecodeGeom {
     const int32_t* r_dev;   // optional: residual row count read at run time (R is then the capacity)
     float* mm;    // [B][Hq][nsplit][2] chunk logit min / max
     float* part;  // [B][Hq][nx][kD + 2] partials (m, l, acc)
+    float* lgt;   // chunked launch: [unit][T][HPB] logits, written by the min/max launch and read by the main
+                  // launch instead of its own K look-ups; NULL: the main launch recomputes them
+    int* cnt;     // chunked launch: [unit] count of the unit's chunks (+ residual unit) that have written their
+                  // partial; the one that finds all the others done merges them
     int B, Hq, Hkv, T, R, S;
     int nsplit, chunk, nx;
     int calib;
@@ -245,6 +252,11 @@ template <int N> __device__ __forceinline__ Vec<N> lds_floats(uint32_t addr) {
     return r;
 }
 
+// A float handed from one workgroup to another inside a launch: device-scope atomic store.
+__device__ __forceinline__ void publish(float* p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 __device__ __forceinline__ uint32_t pack_f16(float a, float b) {
     typedef float f32x2_t __attribute__((ext_vector_type(2)));
     const f32x2_t v = {a, b};
@@ -328,6 +340,12 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
     // A unit without packed tokens or without residual rows aims the unused streams
     // at q (always mapped, at least 256 bytes) and never looks at what comes back.
     const bool has_img = n > 0;
+    // chunked launch with a logits buffer: the min/max launch leaves this chunk's logits there and the main
+    // launch takes them from there - no packed K rows, no table, no look-ups of its own
+    const int64_t unit = bh * static_cast<int64_t>(g.d_ng.div) + hg;
+    V* gl = reinterpret_cast<V*>(g.lgt) + (unit * g.T + t0);
+    const bool from_gl = !MINMAX_ONLY && g.lgt != nullptr && has_img;
+    const bool k_rows = has_img && !from_gl;
     uint32_t q_raw, s_raw, z_raw;
     constexpr bool kVSep = (HPB * kD > kNT - kD);
     uint32_t vs_raw = 0, vz_raw = 0;
@@ -348,10 +366,11 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
         }
     }
     const int64_t code_off = has_img ? (bh * g.T + t0) * NB : 0;   // one offset for both code streams
-    const uint4* ckp = reinterpret_cast<const uint4*>((has_img ? g.ck : static_cast<const uint8_t*>(g.q)) + code_off);
+    const uint4* ckp = reinterpret_cast<const uint4*>(k_rows ? g.ck + code_off : static_cast<const uint8_t*>(g.q));
     const uint4* cvp = reinterpret_cast<const uint4*>((has_img ? g.cv : static_cast<const uint8_t*>(g.q)) + code_off);
     const U4* cvp4 = reinterpret_cast<const U4*>(cvp);
     const int last_u = has_img ? n * NB / 16 - 1 : 0;   // last valid 16-byte unit of either stream
+    const int last_uk = k_rows ? last_u : 0;
     // residual tile: K slice (row = tid / LPR, 128 / LPR elements); V: a wave owns RPW rows of the tile and a
     // lane one channel pair of each of them, so the value products need no fold inside the wave
     constexpr int LPR = L::LPR, NKP = L::NKP, RPW = L::RPW;
@@ -418,7 +437,30 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
 #pragma unroll
     for (int r = 0; r < L::KR; ++r) {
 #pragma unroll
-        for (int i = 0; i < BITS; ++i) kc[r][i] = ckp[min((tid + r * kNT) * BITS + i, last_u)];
+        for (int i = 0; i < BITS; ++i) kc[r][i] = ckp[min((tid + r * kNT) * BITS + i, last_uk)];
+    }
+    // Chunked launch: the chunks' logit min / max, lane s the pair of chunk s for every head (all in flight
+    // together; they are folded across the wave where the calibration needs them), and - with a logits
+    // buffer and the logits in registers - this thread's logits.
+    struct alignas(8) MinMax { float lo, hi; };
+    MinMax mraw[HPB];
+    // REGL: the logits of this thread's tokens, round r = token tid + r * kNT
+    V lg[REGL > 0 ? REGL : 1];
+    if constexpr (!MINMAX_ONLY) {
+        if (g.nsplit > 1 && has_img) {
+#pragma unroll
+            for (int h = 0; h < HPB; ++h) {
+                const MinMax* p = reinterpret_cast<const MinMax*>(g.mm) +
+                                  (static_cast<int64_t>(b) * g.Hq + hq0 + min(h, nh - 1)) * g.nsplit;
+                mraw[h] = p[min(lane, g.nsplit - 1)];
+            }
+        }
+        if constexpr (REGL > 0) {
+            if (from_gl) {
+#pragma unroll
+                for (int rd = 0; rd < REGL; ++rd) lg[rd] = gl[min(tid + rd * kNT, n - 1)];
+            }
+        }
     }
     __syncthreads();
 
@@ -427,8 +469,6 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
     float mn[HPB], mx[HPB];
 #pragma unroll
     for (int h = 0; h < HPB; ++h) { mn[h] = INFINITY; mx[h] = -INFINITY; }
-    // REGL: the logits of this thread's tokens, round r = token tid + r * kNT
-    V lg[REGL > 0 ? REGL : 1];
     // logits (later: calibrated, masked logits) of a token: in its slot, or in the thread's registers
     auto load_logits = [&](int rd, int tt) {
         if constexpr (REGL > 0) return lg[rd];
@@ -461,7 +501,13 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
         for (int r = 0; r < kVEarly; ++r) request_v(r);
     }
 
-    if (n > 0) {
+    if (from_gl) {
+        // (the look-up rounds, which request the rest of the first packed V block as they go, do not run)
+#pragma unroll
+        for (int r = kVEarly; r < kPF; ++r) request_v(r);
+        if constexpr (REGL == 0) for_my_tokens(n, [&](int rd, int tt) { store_logits(rd, tt, gl[tt]); });
+    }
+    if (k_rows) {
         // ---- phase 2: byte table = high-nibble table + low-nibble table ----------------
         // nibble tables: entry (j, half, v) = sum of the per-bit weights v selects; the
         // zero-point sum of the byte position is folded into the high half.
@@ -572,6 +618,9 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                     for (int h = 0; h < HPB; ++h) acc.v[h] += prev.v[h];
                 }
                 if constexpr (!MINMAX_ONLY || P + 1 < L::KPASS) store_logits(rd, tt, acc);
+                if constexpr (MINMAX_ONLY && P + 1 == L::KPASS) {
+                    if (g.lgt) gl[tt] = acc;   // for the main launch
+                }
                 if constexpr (P + 1 == L::KPASS) {
 #pragma unroll
                     for (int h = 0; h < HPB; ++h) { mn[h] = fminf(mn[h], acc.v[h]); mx[h] = fmaxf(mx[h], acc.v[h]); }
@@ -653,7 +702,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
         }
     }
     phase_priority(std::integral_constant<int, 2>{});
-    if (n > 0) {   // one reduction for both: max of (-min, max)
+    if (k_rows) {   // one reduction for both: max of (-min, max)
         float mm2[2 * HPB];
 #pragma unroll
         for (int h = 0; h < HPB; ++h) { mm2[h] = -mn[h]; mm2[HPB + h] = mx[h]; }
@@ -671,6 +720,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                 o[1] = mx[h];
             }
         }
+        if (split == 0 && tid == 0) g.cnt[unit] = 0;   // the main launch counts the unit's partials from 0
         return;
     } else {
         float m_img[HPB];
@@ -716,14 +766,23 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             }
 
             // ---- phase 4: calibration + exp ---------------------------------------------
-            if (g.nsplit > 1) {
+            if (g.nsplit > 1) {   // one fold for both: max of (-min, max) over the chunks
+                float mm2[2 * HPB];
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) {
-                    const float* p = g.mm + (static_cast<int64_t>(b) * g.Hq + hq0 + min(h, nh - 1)) * g.nsplit * 2;
-                    float a = INFINITY, z = -INFINITY;
-                    for (int s = 0; s < g.nsplit; ++s) { a = fminf(a, p[2 * s]); z = fmaxf(z, p[2 * s + 1]); }
-                    mn[h] = a; mx[h] = z;
+                    mm2[h] = -mraw[h].lo;
+                    mm2[HPB + h] = mraw[h].hi;
+                    const MinMax* p = reinterpret_cast<const MinMax*>(g.mm) +
+                                      (static_cast<int64_t>(b) * g.Hq + hq0 + min(h, nh - 1)) * g.nsplit;
+                    for (int s = lane + 64; s < g.nsplit; s += 64) {   // (more than 64 chunks)
+                        const MinMax v = p[s];
+                        mm2[h] = fmaxf(mm2[h], -v.lo);
+                        mm2[HPB + h] = fmaxf(mm2[HPB + h], v.hi);
+                    }
                 }
+                wave_reduce_n<2 * HPB>(mm2, OpMax(), -INFINITY);
+#pragma unroll
+                for (int h = 0; h < HPB; ++h) { mn[h] = -mm2[h]; mx[h] = mm2[HPB + h]; }
             }
             float slope[HPB], tmin[HPB];
 #pragma unroll
@@ -1137,29 +1196,57 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             } else {
                 float* p = g.part + (row * g.nx + split) * (kD + 2);
                 const bool is_img = split < g.nsplit;
-                if (d == 0) { p[0] = is_img ? mi : mr; p[1] = is_img ? li : lr; }
-                p[2 + d] = is_img ? o_img : o_res;
+                if (d == 0) { publish(p, is_img ? mi : mr); publish(p + 1, is_img ? li : lr); }
+                publish(p + 2 + d, is_img ? o_img : o_res);
+            }
+        }
+        if (g.nsplit > 1) {
+            // The unit's chunks (and its residual unit) each leave an (m, l, acc) partial; the workgroup that
+            // finds all the others' already counted combines them.  The partials are device-scope atomic stores
+            // (written through to the level all compute units share, so no cache has to be written back as a
+            // whole): every thread waits for its own stores to complete, the barrier collects the workgroup,
+            // then one thread counts.
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            __builtin_amdgcn_s_waitcnt(0);
+            __syncthreads();
+            int* last = reinterpret_cast<int*>(red);
+            if (tid == 0) *last = __hip_atomic_fetch_add(g.cnt + unit, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == g.nx - 1;
+            __syncthreads();
+            if (*last) {
+                // the reader: one acquire drops this compute unit's and this die's cached copies of what other
+                // dies wrote, after which ordinary loads (issued together, unlike atomic ones) see the partials
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+                if (tid < nh * kD) {
+                    const int h = tid / kD, d = tid % kD;
+                    const int64_t row = static_cast<int64_t>(b) * g.Hq + hq0 + h;
+                    const float* p = g.part + row * g.nx * (kD + 2);
+                    // eight partials at a time, their loads in flight together; running (m, num, den)
+                    float m = -INFINITY, num = 0.f, den = 0.f;
+                    for (int s0 = 0; s0 < g.nx; s0 += 8) {
+                        float ms[8], ls[8], as[8];
+#pragma unroll
+                        for (int k = 0; k < 8; ++k) {
+                            const float* q = p + min(s0 + k, g.nx - 1) * (kD + 2);
+                            ms[k] = q[0]; ls[k] = q[1]; as[k] = q[2 + d];
+                        }
+                        float mb = m;
+#pragma unroll
+                        for (int k = 0; k < 8; ++k) mb = fmaxf(mb, (s0 + k < g.nx) ? ms[k] : -INFINITY);
+                        const float keep = (m == -INFINITY) ? 0.f : __expf(m - mb);
+                        num *= keep; den *= keep;
+#pragma unroll
+                        for (int k = 0; k < 8; ++k) {
+                            const float w = (s0 + k < g.nx && ms[k] != -INFINITY) ? __expf(ms[k] - mb) : 0.f;
+                            den += ls[k] * w;
+                            num += as[k] * w;
+                        }
+                        m = mb;
+                    }
+                    store_elem<DT>(g.out, row * kD + d, num / den);
+                }
             }
         }
     }
-}
-
-// Combine the (m, l, acc) partials of one (batch, q-head) row.  grid (B*Hq), kD threads.
-template <typename DT>
-__global__ void merge_kernel(const float* __restrict__ part, int nx, void* __restrict__ out) {
-    const int64_t row = blockIdx.x;
-    const int d = threadIdx.x;
-    const float* p = part + row * nx * (kD + 2);
-    float m = -INFINITY;
-    for (int s = 0; s < nx; ++s) m = fmaxf(m, p[s * (kD + 2)]);
-    float num = 0.f, den = 0.f;
-    for (int s = 0; s < nx; ++s) {
-        const float ms = p[s * (kD + 2)];
-        const float w = (ms == -INFINITY) ? 0.f : __expf(ms - m);
-        den += p[s * (kD + 2) + 1] * w;
-        num += p[s * (kD + 2) + 2 + d] * w;
-    }
-    store_elem<DT>(out, row * kD + d, num / den);
 }
 
 // Compute units of the current device (a partitioned device reports its own share), asked once per
@@ -1184,7 +1271,7 @@ static inline int ngroups(int G, int hpb) { return (G + hpb - 1) / hpb; }
 
 struct Plan {
     int hpb, nt, regl, nsplit, chunk, nx, cap, lds;
-    size_t ws_mm, ws_part;
+    size_t ws_mm, ws_part, ws_cnt, ws_lgt;   // chunked launch: min / max, partials, counters; logits (optional)
 };
 
 template <int BITS, int HPB, bool VTOK, int NT = 1024, int REGL = 0>
@@ -1222,7 +1309,13 @@ static void plan_for(const cq_decode_args* a, Plan* p) {
     p->lds = L::lds_bytes(p->cap);
     const size_t rows = static_cast<size_t>(a->B) * a->Hq;
     p->ws_mm = nsplit > 1 ? ((rows * nsplit * 2 * sizeof(float) + 255) / 256 * 256) : 0;
-    p->ws_part = nsplit > 1 ? rows * p->nx * (kD + 2) * sizeof(float) : 0;
+    p->ws_part = nsplit > 1 ? (rows * p->nx * (kD + 2) * sizeof(float) + 255) / 256 * 256 : 0;
+    p->ws_cnt = nsplit > 1 ? (static_cast<size_t>(units) * sizeof(int) + 255) / 256 * 256 : 0;
+    // The logits go through a buffer where that is less traffic than the main launch reading the packed K rows
+    // again (4 bytes per head and token against the row's 16 or 32 bytes).  Measured at batch 8 x 32 768 tokens,
+    // four heads per unit: 2 bits 108.6 -> 90.9 us with the buffer, 1 bit (equal bytes) 52.3 -> 54.0 us.
+    const bool hand_over = nsplit > 1 && 16 * BITS > 4 * HPB;
+    p->ws_lgt = hand_over ? static_cast<size_t>(units) * a->T * HPB * sizeof(float) : 0;
 }
 
 static int make_plan(const cq_decode_args* a, Plan* p) {
@@ -1332,7 +1425,9 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
     }
     DecodeGeom gm = g;
     gm.G = G;
-    gm.ncu = (NT == 512 && static_cast<int64_t>(units) * g.nx <= 2 * static_cast<int64_t>(pair_units())) ? pair_units() : 0;
+    // (a main launch that reads its logits back has no look-up phase for the first workgroup to get ahead in:
+    // with the priorities the second one would hold the packed-V loop to itself)
+    gm.ncu = (NT == 512 && !g.lgt && static_cast<int64_t>(units) * g.nx <= 2 * static_cast<int64_t>(pair_units())) ? pair_units() : 0;
     gm.d_ng.set(static_cast<uint32_t>(ngroups(G, HPB)));
     gm.d_nx.set(static_cast<uint32_t>(g.nx));
     gm.d_hkv.set(static_cast<uint32_t>(g.Hkv));
@@ -1348,11 +1443,6 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
     }
     hipLaunchKernelGGL(kmain, dim3(units * g.nx), dim3(NT), p.lds, st, gm);
     CQ_LAUNCH_CHECK();
-    if (g.nsplit > 1) {
-        hipLaunchKernelGGL(merge_kernel<DT>, dim3(static_cast<unsigned>(g.B) * g.Hq), dim3(kD), 0, st, g.part, g.nx,
-                           g.out);
-        CQ_LAUNCH_CHECK();
-    }
     return CQ_OK;
 }
 
@@ -1417,7 +1507,12 @@ static int decode_entry(const cq_decode_args* a, void* workspace, size_t workspa
     if (a->R > 0 && (!aligned16(a->k_res) || !aligned16(a->v_res) || (a->res_stride_b % 8) ||
                      (a->res_stride_h % 8) || (a->res_stride_r % 8)))
         return CQ_ERR_ALIGN;
-    const size_t need = p.ws_mm + p.ws_part;
+    // the logits buffer is the last part of the workspace; the static scratch does without it when it
+    // does not fit (the main launch then recomputes the logits)
+    const size_t need_min = p.ws_mm + p.ws_part + p.ws_cnt;
+    bool with_logits = p.ws_lgt > 0;
+    if (static_scratch && need_min + p.ws_lgt > kScratchBytes) with_logits = false;
+    const size_t need = need_min + (with_logits ? p.ws_lgt : 0);
     if (static_scratch) {
         if (need > kScratchBytes) return CQ_ERR_SCRATCH_LIMIT;
         workspace = nullptr;
@@ -1439,6 +1534,8 @@ static int decode_entry(const cq_decode_args* a, void* workspace, size_t workspa
     g.out = a->out;
     g.mm = static_cast<float*>(workspace);
     g.part = need ? reinterpret_cast<float*>(static_cast<char*>(workspace) + p.ws_mm) : nullptr;
+    g.cnt = need ? reinterpret_cast<int*>(static_cast<char*>(workspace) + p.ws_mm + p.ws_part) : nullptr;
+    g.lgt = with_logits ? reinterpret_cast<float*>(static_cast<char*>(workspace) + need_min) : nullptr;
     g.B = a->B; g.Hq = a->Hq; g.Hkv = a->Hkv; g.T = a->T; g.R = a->R; g.S = a->sprompt_len;
     g.nsplit = p.nsplit; g.chunk = p.chunk; g.nx = p.nx;
     g.calib = a->calibrate; g.off_max = a->calib_off_max; g.off_min = a->calib_off_min;
@@ -1458,7 +1555,7 @@ extern "C" {
 size_t cq_decode_attn_workspace(const cq_decode_args* args) {
     cq::Plan p;
     if (cq::make_plan(args, &p) != CQ_OK) return 0;
-    return p.ws_mm + p.ws_part;
+    return p.ws_mm + p.ws_part + p.ws_cnt + p.ws_lgt;
 }
 
 int cq_decode_attn_plan(const cq_decode_args* args, cq_decode_plan* plan) {
@@ -1470,7 +1567,7 @@ int cq_decode_attn_plan(const cq_decode_args* args, cq_decode_plan* plan) {
     plan->heads_per_unit = p.hpb;
     plan->chunks = p.nsplit;
     plan->chunk_tokens = args->T > 0 ? p.chunk : 0;
-    plan->launches = p.nsplit > 1 ? 3 : 1;
+    plan->launches = p.nsplit > 1 ? 2 : 1;
     plan->lds_bytes = p.lds;
     plan->register_logits = p.regl;
     return CQ_OK;

@@ -246,15 +246,18 @@ int cq_decode_attn(const cq_decode_args* args, cq_stream_t stream);
  * outputs and temporaries with torch on every call.  Same arguments and the
  * same kernels as cq_decode_attn, except that args->workspace /
  * workspace_bytes are ignored: the scratch of the chunked path (per-chunk
- * logit min / max and the flash-decoding partials, what
- * cq_decode_attn_workspace() sizes) lives in a static device array of
- * cq_decode_attn_static_limit() bytes (8 MiB) inside the library; every GPU
- * the library runs on holds its own copy until the process ends.  A request
- * whose plan needs more returns CQ_ERR_SCRATCH_LIMIT and launches nothing
- * (batch 8 x 32 768 tokens needs 1.2 MiB).  The call allocates and frees
- * nothing and does not synchronise.  Nothing in the scratch has to start at
- * zero: every word a launch reads was written by an earlier launch of the
- * same call.  All calls on one GPU share that GPU's array, so two calls that
+ * logit min / max, the flash-decoding partials and their counters, and - where
+ * the plan hands the first launch's logits to the second through a buffer
+ * (2 bits, or fewer than four heads per unit) and it fits beside them - those)
+ * lives in a static device array of cq_decode_attn_static_limit() bytes
+ * (8 MiB) inside the library; every GPU the library runs on holds its own
+ * copy until the process ends.  When the logits do not fit, the second launch
+ * recomputes them (same results, more work).  A request whose plan needs more
+ * than the limit even so returns CQ_ERR_SCRATCH_LIMIT and launches nothing
+ * (batch 8 x 32 768 tokens needs 1.2 MiB; at 2 bits 33 MiB more with the logits).
+ * The call allocates and frees nothing and does not synchronise.  Nothing in
+ * the scratch has to start at zero: every word a launch reads was written by
+ * an earlier launch of the same call (the first launch clears the counters).  All calls on one GPU share that GPU's array, so two calls that
  * may overlap on one GPU (different streams, or one stream per host thread)
  * race on it: keep them on one stream, or give the overlapping ones
  * cq_decode_attn with workspaces of their own. */
@@ -270,9 +273,9 @@ int cq_decode_attn_static(const cq_decode_args* args, cq_stream_t stream);
 typedef struct cq_decode_plan {
     int threads;          /* threads per workgroup: 1024, or 512 with two workgroups per compute unit */
     int heads_per_unit;   /* query heads served by one workgroup (they share a kv head) */
-    int chunks;           /* token chunks per (batch, kv head, head group); > 1: min/max launch + main launch + merge */
+    int chunks;           /* token chunks per (batch, kv head, head group); > 1: logits + min/max launch, then the main launch (which also merges) */
     int chunk_tokens;     /* packed tokens per chunk */
-    int launches;         /* 1 or 3 */
+    int launches;         /* 1 or 2 */
     int lds_bytes;        /* dynamic LDS of the main launch */
     int register_logits;  /* > 0: a thread keeps the logits of up to this many of its tokens in registers (fp32)
                            * and the token slots in LDS hold only exp(.) as fp16; 0: fp32 logits wait in the slots */

@@ -28,7 +28,7 @@ def test_library_loads_and_exports_every_declared_symbol():
 def test_decode_launch_plan_is_a_function_of_the_shape():
     """`cq_decode_attn_plan` (host only): which launch a shape gets.  Two 512-thread workgroups per compute
     unit need a layout within half of the 160 KB LDS and more units of work than the 256 compute units;
-    logits kept in registers only at 1 bit with four heads per unit; chunked shapes take three launches."""
+    logits kept in registers only at 1 bit with four heads per unit; chunked shapes take two launches."""
     from calibquant_amd import _lib
     lib = _lib.load()
 
@@ -48,17 +48,17 @@ def test_decode_launch_plan_is_a_function_of_the_shape():
     assert (two_bit["threads"], two_bit["register_logits"]) == (512, 8) and two_bit["lds_bytes"] <= 80 * 1024
     assert plan(32, 32, 8, 3328, 128, bits=2)["threads"] == 1024
     assert plan(64, 32, 8, 3328, 128, v_mode=1)["threads"] == 1024
-    assert plan(64, 32, 8, 3328, 128, force_splits=2) == dict(plan(64, 32, 8, 3328, 128, force_splits=2), threads=1024, launches=3)
+    assert plan(64, 32, 8, 3328, 128, force_splits=2) == dict(plan(64, 32, 8, 3328, 128, force_splits=2), threads=1024, launches=2)
     two = plan(128, 16, 8, 3328, 128)                        # two heads per unit: paired, fp32 logits
     assert (two["threads"], two["heads_per_unit"], two["register_logits"]) == (512, 2, 0)
     long = plan(8, 32, 8, 32768, 0)                          # chunked: the chunks are the units
-    assert long["launches"] == 3 and long["threads"] == 512 and long["chunks"] * long["chunk_tokens"] >= 32768
+    assert long["launches"] == 2 and long["threads"] == 512 and long["chunks"] * long["chunk_tokens"] >= 32768
     assert long["lds_bytes"] <= 80 * 1024
     big = plan(16, 48, 8, 9984, 64)     # six heads per kv head: two units of four (the second half padding); one launch
     assert (big["threads"], big["heads_per_unit"], big["launches"], big["register_logits"]) == (1024, 4, 1, 10)   # logits in registers
     assert big["lds_bytes"] <= 160 * 1024
     tok = plan(16, 48, 8, 9984, 64, v_mode=1)               # per-token values: padded four-head units too, chunked (16-byte slots)
-    assert (tok["heads_per_unit"], tok["threads"], tok["register_logits"]) == (4, 1024, 0) and tok["launches"] == 3
+    assert (tok["heads_per_unit"], tok["threads"], tok["register_logits"]) == (4, 1024, 0) and tok["launches"] == 2
     a = _lib.DecodeArgs()
     assert lib.cq_decode_attn_plan(ctypes.byref(a), None) < 0
     assert lib.cq_decode_attn_plan(ctypes.byref(a), ctypes.byref(_lib.DecodePlan())) < 0   # all-zero arguments
@@ -67,7 +67,7 @@ def test_decode_launch_plan_is_a_function_of_the_shape():
 def test_decode_launch_plan_invariants_over_random_shapes():
     """Whatever the shape, the plan stays inside what the kernels assume: LDS within the device's 160 KB (half of
     it for a 512-thread workgroup), chunks that cover T, register-resident logits only for chunks that fit the
-    rounds a thread keeps, three launches and a workspace exactly when T is chunked."""
+    rounds a thread keeps, two launches and a workspace exactly when T is chunked."""
     from calibquant_amd import _lib
     lib = _lib.load()
     rng = np.random.default_rng(11)
@@ -90,7 +90,7 @@ def test_decode_launch_plan_invariants_over_random_shapes():
         assert p.chunks >= 1 and p.chunks * p.chunk_tokens >= a.T, shape
         assert p.chunk_tokens % 64 == 0, shape
         assert p.register_logits == 0 or p.chunk_tokens <= p.register_logits * p.threads, shape
-        assert p.launches == (3 if p.chunks > 1 else 1), shape
+        assert p.launches == (2 if p.chunks > 1 else 1), shape
         assert (lib.cq_decode_attn_workspace(ctypes.byref(a)) > 0) == (p.chunks > 1), shape
         if a.v_mode == 1:
             assert p.threads == 1024 and p.register_logits == 0, shape

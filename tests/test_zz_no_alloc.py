@@ -1,6 +1,6 @@
 """`cq_decode_attn_static`, the entry point that allocates nothing: its scratch (per-chunk logit
-min / max and flash-decoding partials of the chunked path) is a static device buffer inside the
-library.  Called through the C ABI on two calls in a row, the second with a smaller input, and
+min / max, flash-decoding partials and - when they fit - the logits the first launch hands to the
+second) is a static device buffer inside the library.  Called through the C ABI on two calls in a row, the second with a smaller input, and
 compared with `cq_decode_attn` (caller-provided workspace) and with the oracle."""
 import ctypes as C
 
@@ -36,7 +36,7 @@ def test_static_scratch_entry_point_two_calls_in_a_row():
     lib = _lib.load()
     assert lib.cq_decode_attn_static_limit() == 8 << 20
     stream = torch.cuda.current_stream().cuda_stream
-    # first call: 4 x 12 000 tokens + 50 window rows (chunked: min/max launch, main launch, merge);
+    # first call: 4 x 12 000 tokens + 50 window rows (chunked: logits + min/max launch, main launch);
     # second call: a smaller input (2 x 9 000 tokens, no window) that reuses the same scratch
     for (B, T, R, S, bits, seed) in ((4, 12000, 50, 7, 1, 401), (2, 9000, 0, 0, 1, 402), (2, 5000, 30, 0, 2, 403)):
         Hq, Hkv = 32, 8
@@ -60,6 +60,27 @@ def test_static_scratch_entry_point_two_calls_in_a_row():
                                   c["kr"][:, :, :R], c["vr"][:, :, :R], S, bits)
         err = np.abs(to_np(out_st) - want)
         assert err.max() < 1e-2 and err.mean() < 1e-3, (T, float(err.max()), float(err.mean()))
+    # 2 x 32 768 tokens at 2 bits: the logits the first launch would hand to the second are alone beyond the
+    # static buffer, so the static entry point's main launch recomputes them while the workspace entry point
+    # reads them back - same bits either way
+    B, Hq, Hkv, T, R, S = 2, 32, 8, 32768, 40, 5
+    c = make_case(B, Hq, Hkv, 128, T, R, 2, "bf16", seed=405, outlier_kind="student")
+    g = case_to_gpu(c, "bf16")
+    out_ws = torch.zeros((B, Hq, 128), dtype=torch.bfloat16, device="cuda")
+    out_st = torch.zeros_like(out_ws)
+    a = _args(_lib, g, B, Hq, Hkv, T, R, S, 2, out_ws)
+    need = lib.cq_decode_attn_workspace(C.byref(a))
+    assert need > lib.cq_decode_attn_static_limit()
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    a.workspace, a.workspace_bytes = ws.data_ptr(), need
+    assert lib.cq_decode_attn(C.byref(a), stream) == 0
+    b = _args(_lib, g, B, Hq, Hkv, T, R, S, 2, out_st)
+    assert lib.cq_decode_attn_static(C.byref(b), stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out_ws, out_st)
+    want = O.decode_attention(c["q"], c["ck"], c["cv"], c["sk"], c["zk"], c["sv"], c["zv"], c["kr"], c["vr"], S, 2)
+    err = np.abs(to_np(out_st) - want)
+    assert err.max() < 1e-2 and err.mean() < 1e-3, (T, float(err.max()), float(err.mean()))
     # a single-launch shape needs no scratch and works as well
     c = make_case(2, 32, 8, 128, 700, 20, 1, "bf16", seed=404)
     g = case_to_gpu(c, "bf16")
