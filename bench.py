@@ -490,6 +490,13 @@ def main():
 
     shape = WORKLOADS[a.workload]
     B, Hq, Hkv, D, T, R, S = shape
+    if a.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     if a.only in ("prefill", "prefill-contiguous"):
         print(json.dumps(prefill_leg(torch, ops, shape, a.bits, a.steps, a.warmup, a.only == "prefill-contiguous")))
         return
@@ -499,12 +506,6 @@ def main():
         return
     calls = [ops.DecodeCall(s["q"], s["ck"], s["cv"], s["sk"], s["zk"], s["sv"], s["zv"], s["kr"], s["vr"],
                             sprompt_len=S, bits=a.bits) for s in sets]
-    if a.copy_calibration:
-        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
     ms = time_calls(torch, calls, a.steps, a.warmup, a.settle_ms)
     plan = calls[0].plan()
     nbytes = algorithmic_bytes(B, Hq, Hkv, D, T, R, a.bits)

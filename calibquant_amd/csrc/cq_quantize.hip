@@ -19,6 +19,9 @@
 // only compares - the per-element IEEE division would otherwise bound the pass.
 #include "cq_common.h"
 
+#include <mutex>
+#include <vector>
+
 #pragma clang fp contract(off)
 
 namespace cq {
@@ -403,6 +406,9 @@ constexpr int kFThreads = 1024;
 constexpr int kFRows = 13;                  // rows per thread at most (13 x 256 = 12 tiles + thumbnail of 256 tokens)
 constexpr int kFMaxT = kFRows * (kFThreads / 4);
 constexpr int kFGrid = 256;                 // workgroups of the persistent launch (one per compute unit)
+// rows per thread of the next slice that are staged in LDS (16 KB each for the workgroup)
+// (not with the rotary embedding fused in: that instantiation has no registers to spare for the addresses)
+constexpr int fused_stage_rows(int nr, bool rope) { return (nr > 8 && !rope) ? 8 : 0; }
 
 // Rotary embedding fused into the pass (ROPE): x is the un-rotated key block; every row is rotated as it
 // arrives - rnd(rnd(x * cos) + rotate_half(x) * sin), the arithmetic of the ops the reference runs on the
@@ -430,6 +436,12 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
     __shared__ __attribute__((aligned(16))) float part_mn[32][kFThreads / 16];   // [channel][wave * 4 + row of 16 lanes]
     __shared__ __attribute__((aligned(16))) float part_mx[32][kFThreads / 16];
     __shared__ float s_s[32], s_z[32], s_thr[3][32];
+    // NP rows per thread of the NEXT slice travel through LDS: they are requested as soon as this slice's min / max
+    // fold has read the registers - global-to-LDS loads that need no register to land in - so HBM stays busy
+    // through the statistics and threshold phases, in which nothing else is in flight; the emit then refills those
+    // rows' registers from LDS and only the other NR - NP rows from memory.
+    constexpr int NP = fused_stage_rows(NR, ROPE);
+    extern __shared__ __attribute__((aligned(16))) unsigned char stage[];   // [NP][thread][16 bytes]
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int q4 = tid & 3, row = tid >> 2;
     // A workgroup walks slices blockIdx.x, blockIdx.x + gridDim.x, ... (gridDim.x is a multiple
@@ -550,6 +562,20 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
             k_umax[w] = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(US2, k_umax[w]), __builtin_bit_cast(US2, r)));
         }
     }
+    if constexpr (NP > 0) {
+        if (has_next) {
+            // lane l of a wave lands at the wave's base + 16 l: thread tid's piece of row i at stage[i][tid]
+            const int wvu = __builtin_amdgcn_readfirstlane(wv);
+#pragma unroll
+            for (int i = 0; i < NP; ++i)
+                __builtin_amdgcn_global_load_lds(
+                    reinterpret_cast<const __attribute__((address_space(1))) void*>(
+                        reinterpret_cast<uintptr_t>(next_base + row_offset(i * (kFThreads / 4) + row_i))),
+                    reinterpret_cast<__attribute__((address_space(3))) void*>(
+                        static_cast<uint32_t>(reinterpret_cast<uintptr_t>(stage + (i * kFThreads + wvu * 64) * 16))),
+                    16, 0, 0);
+        }
+    }
     float mn[8], mx[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -635,7 +661,18 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
         for (int k = 0; k < L; ++k) th[k][j] = s_thr[k][q4 * 8 + j];
     constexpr int nb = 128 * BITS / 8;   // bytes per packed row
 #pragma unroll
-    for (int i = 0; i < NR; ++i) {
+    for (int e = 0; e < NR; ++e) {
+        // the rows refilled from memory go first (their loads then have the rest of the emit to land), the
+        // staged rows after them
+        const int i = (e + NP) % NR;
+        if constexpr (NP > 0) {
+            if (e == NR - NP) {
+                // Every staged piece has landed once at most NR - NP younger memory operations are outstanding
+                // (the refills just issued; stores issued since only make the wait stricter).  A thread reads
+                // back exactly the bytes its own lane requested, so no barrier is needed.
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NR - NP) : "memory");
+            }
+        }
         const int t = i * (kFThreads / 4) + row_i;
         // (the empty statement keeps the compiler from carrying the unpacked floats of the
         // min/max pass over to here: that would double the registers the slice needs)
@@ -703,9 +740,45 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
             }
         }
         // the row is packed: its registers take the same row of the next slice
-        if (has_next) v[i] = *reinterpret_cast<const U4*>(next_base + row_offset(t));
+        if (has_next) {
+            if (i < NP) v[i] = *reinterpret_cast<const U4*>(stage + (i * kFThreads + tid) * 16);
+            else v[i] = *reinterpret_cast<const U4*>(next_base + row_offset(t));
+        }
     }
     }
+}
+
+// Raises a kernel's dynamic-LDS limit (the default stops at 64 KB); asked of the runtime once per kernel and device.
+static int allow_dynamic_lds(const void* kernel, int bytes) {
+    struct Done { const void* k; uint64_t devices; };
+    static std::mutex mu;
+    static std::vector<Done> done;
+    int dev = 0;
+    CQ_HIP_CHECK(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(mu);
+    for (auto& d : done)
+        if (d.k == kernel) {
+            if (d.devices >> (dev & 63) & 1) return CQ_OK;
+            CQ_HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+            d.devices |= 1ull << (dev & 63);
+            return CQ_OK;
+        }
+    CQ_HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+    done.push_back({kernel, 1ull << (dev & 63)});
+    return CQ_OK;
+}
+
+template <typename DT, int BITS, int NR, bool ROPE>
+static int launch_fused(dim3 grid, hipStream_t st, const uint16_t* xp, const QuantGeom& g, float clip, uint16_t* sp,
+                        uint16_t* zp, uint8_t* codes, const RopeArgs& ra) {
+    constexpr int lds = fused_stage_rows(NR, ROPE) * kFThreads * 16;
+    auto kf = fused_pack_kernel<DT, BITS, NR, ROPE>;
+    if (lds) {
+        const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kf), lds);
+        if (rc != CQ_OK) return rc;
+    }
+    hipLaunchKernelGGL(kf, grid, dim3(kFThreads), lds, st, xp, g, clip, sp, zp, codes, ra);
+    return CQ_OK;
 }
 
 // true if the shape goes through the one-pass kernel (x read once, slice by slice in registers)
@@ -731,10 +804,11 @@ static int run_quant(const void* x, QuantGeom g, int bits, float clip, uint8_t* 
         const dim3 fgrid(static_cast<unsigned>(nsl < kFGrid ? nsl : kFGrid));
         const int nr = (g.T + kFThreads / 4 - 1) / (kFThreads / 4);
         const RopeArgs ra = rope ? *rope : RopeArgs{};
-#define CQ_FUSED(B_, N_)                                                                                              \
-        do {                                                                                                          \
-            if (rope) hipLaunchKernelGGL((fused_pack_kernel<DT, B_, N_, true>), fgrid, dim3(kFThreads), 0, st, xp, g, clip, sp, zp, codes, ra);  \
-            else hipLaunchKernelGGL((fused_pack_kernel<DT, B_, N_, false>), fgrid, dim3(kFThreads), 0, st, xp, g, clip, sp, zp, codes, ra);      \
+#define CQ_FUSED(B_, N_)                                                                          \
+        do {                                                                                      \
+            const int rc = rope ? launch_fused<DT, B_, N_, true>(fgrid, st, xp, g, clip, sp, zp, codes, ra)   \
+                                : launch_fused<DT, B_, N_, false>(fgrid, st, xp, g, clip, sp, zp, codes, ra); \
+            if (rc != CQ_OK) return rc;                                                           \
         } while (0)
         if (bits == 1) {
             if (nr <= 4) CQ_FUSED(1, 4); else if (nr <= 8) CQ_FUSED(1, 8); else CQ_FUSED(1, 13);
