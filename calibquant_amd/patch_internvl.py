@@ -182,10 +182,13 @@ def forward_internlm2_calibquant(self, hidden_states: torch.Tensor, attention_ma
         kv_seq_len += past_key_value[0].shape[-2] + T                               # patch_internvl.py:246-251
     cos, sin = self.rotary_emb(value_states, seq_len=kv_seq_len)
     # Prefill on the GPU: the rotary embedding runs in HIP kernels with the rounding of the reference's op
-    # chain - queries and the keys outside the image block in `cq_rope_rows`, the image block of the keys
-    # inside the quantise-and-pack pass itself (`cq_rope_quantize_pack`: the un-rotated keys are read once,
-    # the rotated rows written once and quantised from the registers).  The reference rotates the whole
-    # tensors with a chain of torch ops first (patch_internvl.py:258-260) and quantises afterwards (:295-297).
+    # chain (`cq_rope_rows` for queries and keys), then the image block of the rotated keys is quantised.
+    # The reference rotates the whole tensors with a chain of torch ops first (patch_internvl.py:258-260) and
+    # quantises afterwards (:295-297).  With `cq_fused_rope` set on the module the image block of the keys is
+    # rotated inside the quantise-and-pack pass instead (`cq_rope_quantize_pack`: un-rotated keys read once,
+    # rotated rows written once, quantised from the registers) - same bits, one launch fewer, but slower at the
+    # benchmark shape (348 against 309 us: a slice then reads two 32-byte pieces per row instead of one of 64,
+    # which HBM serves as 64-byte fetches), so it is not the default.
     hip_rope = (q_len > 1 and qkv.is_cuda and qkv.dtype in (torch.bfloat16, torch.float16) and D == 128
                 and position_ids is not None and position_ids.is_cuda and position_ids.dtype == torch.int64
                 and tuple(position_ids.shape) == (bsz, q_len))
@@ -216,7 +219,7 @@ def forward_internlm2_calibquant(self, hidden_states: torch.Tensor, attention_ma
             raise CalibQuantError(f"prompt of {q_len} tokens is shorter than sprompt_len + image tokens = {S + T}")
         self._cq_call = None
         self.__dict__.pop("_cq_step", None)
-        fused_rope = hip_rope and 0 < T <= ops.ROPE_FUSED_MAX_T
+        fused_rope = hip_rope and 0 < T <= ops.ROPE_FUSED_MAX_T and bool(getattr(self, "cq_fused_rope", False))
         if hip_rope:
             if fused_rope:      # image block: rotated inside the quantiser; the rows around it on their own
                 ck, ks, kz = ops.rope_quantize_pack(k_raw[:, S:S + T], cos, sin, position_ids[:, S:S + T],

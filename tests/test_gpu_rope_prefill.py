@@ -103,3 +103,36 @@ def test_rope_quantize_pack_refuses_what_the_one_pass_kernel_cannot_hold(ops):
     cos, sin = _tables(4100, 128, "bf16")
     with pytest.raises(CalibQuantError):
         ops.rope_quantize_pack(x, cos, sin, 0, torch.empty_like(x), 1, 0.5)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_attention_prefill_same_state_through_every_rotary_path(dtype):
+    """The patched attention's prefill with the rotary embedding (a) in `cq_rope_rows` followed by the
+    quantiser (the default), (b) fused into the quantiser (`cq_fused_rope`), (c) as the chain of torch ops
+    (forced by int32 position ids): the packed codes, statistics and window rows are the same bits; the
+    attention output of (a) and (b) is identical."""
+    from calibquant_amd import patch_internvl as pi
+    from calibquant_amd.internlm2 import InternLM2Attention, InternLM2Config
+    cfg = InternLM2Config.tiny()
+    B, S, T, TXT = 2, 5, 700, 11
+    N = S + T + TXT
+    got = []
+    for mode in ("rows", "fused", "torch"):
+        torch.manual_seed(21)
+        att = InternLM2Attention(cfg).cuda().to(dtype)
+        att.cq_sprompt_len, att.cq_image_token_num = S, T
+        att.cq_fused_rope = mode == "fused"
+        x = torch.randn(B, N, cfg.hidden_size, device="cuda", dtype=dtype)
+        pos = torch.arange(N, device="cuda")[None].expand(B, N)
+        with torch.no_grad():
+            out, _, past = pi.forward_internlm2_calibquant(att, x, None, pos.int() if mode == "torch" else pos, None,
+                                                           False, True)
+        got.append((att.encoded_features_k.clone(), att.encoded_features_v.clone(), [t.clone() for t in att._cq_stats],
+                    past[0].clone(), past[1].clone(), out.clone()))
+    for other in (1, 2):
+        assert torch.equal(got[0][0], got[other][0]) and torch.equal(got[0][1], got[other][1])
+        for a, b in zip(got[0][2], got[other][2]):
+            assert torch.equal(a, b)
+        if dtype == torch.bfloat16 or other == 1:   # (torch's fp16 addcmul rounds once: window rows may differ in the last bit)
+            assert torch.equal(got[0][3], got[other][3]) and torch.equal(got[0][4], got[other][4])
+    assert torch.equal(got[0][5], got[1][5])
