@@ -449,9 +449,10 @@ def model_leg(torch, batch=64, tiles=13, sys_len=41, text_len=23, new_tokens=128
         run_graph("kv_1bit", True)
     finally:
         InternLM2Attention.forward, InternVLChatStandIn.generate = fp_forward, fp_generate
-    res["note"] = ("kv_1bit_decode_tok_s: decode step replayed as a HIP graph; *_eager_*: eager host loop "
-                   "(1-bit: bound by per-layer launch overhead; fp16: torch SDPA, bound by that attention kernel); "
-                   "fp16_kv_own_kernel_*: full-precision cache through this library's attention kernel, HIP graph")
+    res["note"] = ("kv_1bit_decode_tok_s: decode step replayed as a HIP graph; *_eager_*: eager host loop through the "
+                   "patched forward (1-bit: one call into the host shim per layer and token; fp16: torch SDPA, bound by "
+                   "that attention kernel); fp16_kv_own_kernel_*: full-precision cache through this library's attention "
+                   "kernel, HIP graph")
     return res
 
 

@@ -564,16 +564,32 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
     }
     if constexpr (NP > 0) {
         if (has_next) {
-            // lane l of a wave lands at the wave's base + 16 l: thread tid's piece of row i at stage[i][tid]
-            const int wvu = __builtin_amdgcn_readfirstlane(wv);
+            // lane l of a wave lands at the wave's base + 16 l: thread tid's piece of row i at stage[i][tid].
+            // Written as assembly: the compiler waits for a global-to-LDS load it knows of before the next LDS
+            // instruction of any kind, which would take the loads out of flight again at once.  The fold's
+            // results are operands of the first statement only to place the loads after the fold, i.e. after the
+            // compiler's own wait for the rows that came through registers; unknown to the compiler, the loads
+            // can only make its later vector-memory waits stricter, never weaker, and the wait before the
+            // staged pieces are read back is written out below.
+            const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(stage)) +
+                                  static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(wv)) * 1024u;
 #pragma unroll
-            for (int i = 0; i < NP; ++i)
-                __builtin_amdgcn_global_load_lds(
-                    reinterpret_cast<const __attribute__((address_space(1))) void*>(
-                        reinterpret_cast<uintptr_t>(next_base + row_offset(i * (kFThreads / 4) + row_i))),
-                    reinterpret_cast<__attribute__((address_space(3))) void*>(
-                        static_cast<uint32_t>(reinterpret_cast<uintptr_t>(stage + (i * kFThreads + wvu * 64) * 16))),
-                    16, 0, 0);
+            for (int i = 0; i < NP; ++i) {
+                const uint32_t off = row_offset(i * (kFThreads / 4) + row_i);
+                const uint32_t ldsa = lds0 + static_cast<uint32_t>(i) * (kFThreads * 16);
+                if (i == 0)
+                    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %2"
+                                 :
+                                 : "v"(off), "s"(ldsa), "s"(next_base), "v"(k_smax[0]), "v"(k_smax[1]), "v"(k_smax[2]),
+                                   "v"(k_smax[3]), "v"(k_umin[0]), "v"(k_umin[1]), "v"(k_umin[2]), "v"(k_umin[3]),
+                                   "v"(k_umax[0]), "v"(k_umax[1]), "v"(k_umax[2]), "v"(k_umax[3])
+                                 : "memory", "m0");
+                else
+                    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %2"
+                                 :
+                                 : "v"(off), "s"(ldsa), "s"(next_base)
+                                 : "memory", "m0");
+            }
         }
     }
     float mn[8], mx[8];
