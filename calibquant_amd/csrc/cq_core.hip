@@ -7,7 +7,7 @@ thread_local int g_last_hip_error = 0;
 
 extern "C" {
 
-int cq_version(void) { return 104; }   // 104: cq_rope_quantize_pack, cq_rope_rows; 103: cq_decode_attn_static; 102: lut_len argument of the look-up vec-mats, cq_quant_tensor
+int cq_version(void) { return 105; }   // 105: chunked decode in two launches (merge inside the main launch; workspace holds counters and, where used, logits); 104: cq_rope_quantize_pack, cq_rope_rows; 103: cq_decode_attn_static; 102: lut_len argument of the look-up vec-mats, cq_quant_tensor
 
 const char* cq_strerror(int status) {
     switch (status) {

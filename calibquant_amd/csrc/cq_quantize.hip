@@ -570,7 +570,8 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
             // results are operands of the first statement only to place the loads after the fold, i.e. after the
             // compiler's own wait for the rows that came through registers; unknown to the compiler, the loads
             // can only make its later vector-memory waits stricter, never weaker, and the wait before the
-            // staged pieces are read back is written out below.
+            // staged pieces are read back is written out below.  (m0, the LDS base of such a load, has no other
+            // use in this kernel; the compiler reserves it and does not accept it as a clobber.)
             const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(stage)) +
                                   static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(wv)) * 1024u;
 #pragma unroll
@@ -583,12 +584,12 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
                                  : "v"(off), "s"(ldsa), "s"(next_base), "v"(k_smax[0]), "v"(k_smax[1]), "v"(k_smax[2]),
                                    "v"(k_smax[3]), "v"(k_umin[0]), "v"(k_umin[1]), "v"(k_umin[2]), "v"(k_umin[3]),
                                    "v"(k_umax[0]), "v"(k_umax[1]), "v"(k_umax[2]), "v"(k_umax[3])
-                                 : "memory", "m0");
+                                 : "memory");
                 else
                     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %2"
                                  :
                                  : "v"(off), "s"(ldsa), "s"(next_base)
-                                 : "memory", "m0");
+                                 : "memory");
             }
         }
     }

@@ -100,11 +100,14 @@ def test_quant_and_encode_operators(ops, bits, dtype):
         assert torch.equal(enc, codes)
 
 
+@pytest.mark.parametrize("B", [4, 64])
 @pytest.mark.parametrize("bits", [1, 2])
-def test_quantize_pack_matches_torch_device_op_chain(ops, bits):
+def test_quantize_pack_matches_torch_device_op_chain(ops, bits, B):
     """torch's own device kernels, run op by op on the 16-bit tensor, are the
-    primitives the reference executes (calibquant.py:27-36)."""
-    B, T, H, D = 4, 3328, 8, 128
+    primitives the reference executes (calibquant.py:27-36).  At batch 64 (the benchmark's prefill
+    tensor) every workgroup of the one-pass kernel walks eight slices, the later ones with part of
+    their rows staged through LDS."""
+    T, H, D = 3328, 8, 128
     g = torch.Generator(device="cuda").manual_seed(5)
     x = torch.randn((B, T, H, D), generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
     clip = CLIPS[bits][0]
