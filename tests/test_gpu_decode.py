@@ -386,3 +386,29 @@ def test_decode_attn_rejects_bad_arguments(ops):
     with pytest.raises(CalibQuantError):
         ops.decode_attn(g["q"][:, :, :64].contiguous(), g["ck"], g["cv"], g["sk"], g["zk"], g["sv"], g["zv"],
                         g["kr"], g["vr"])
+
+
+@pytest.mark.parametrize("case", [(2, 16, 8, 20000, 50, 3, 1), (2, 8, 8, 20000, 0, 0, 1), (1, 32, 8, 20000, 33, 5, 2),
+                                  (1, 16, 8, 20000, 33, 0, 2)], ids=lambda c: "-".join(str(x) for x in c))
+def test_decode_attn_chunked_with_the_logits_buffer(ops, case):
+    """Chunked launches whose first launch hands the logits to the second through the workspace (a packed K row
+    of more bytes than the logits: 2 bits, or fewer than four heads per unit), against the oracle.  (Four-head
+    units at 1 bit recompute their logits: `test_long_context_batch_8_kv_32768` and the chunked cases above.)"""
+    B, Hq, Hkv, T, R, S, bits = case
+    c = make_case(B, Hq, Hkv, 128, T, max(R, 1), bits, "bf16", seed=500 + Hq + bits, outlier_kind="student")
+    g = case_to_gpu(c, "bf16")
+    call = ops.DecodeCall(g["q"], g["ck"], g["cv"], g["sk"], g["zk"], g["sv"], g["zv"], g["kr"] if R else None,
+                          g["vr"] if R else None, sprompt_len=S, bits=bits)
+    plan = call.plan()
+    assert plan["chunks"] > 1 and plan["launches"] == 2
+    units = B * Hkv * ((Hq // Hkv + plan["heads_per_unit"] - 1) // plan["heads_per_unit"])
+    assert call.workspace_bytes >= units * T * plan["heads_per_unit"] * 4      # the logits are part of it
+    out = call.run()
+    torch.cuda.synchronize()
+    want = O.decode_attention(c["q"], c["ck"], c["cv"], c["sk"], c["zk"], c["sv"], c["zv"],
+                              c["kr"][:, :, :R] if R else None, c["vr"][:, :, :R] if R else None, S, bits)
+    _check(to_np(out), want)
+    # twice in a row on the same workspace: the counters start from zero again
+    out2 = call.run()
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
