@@ -233,7 +233,7 @@ def side_legs(torch, ops, shape, bits, sets, settle_ms=0.0, only_token=False):
         res["prefill_quantize_pack"] = prefill_leg(torch, ops, shape, bits)
     proj = torch.randn((B, T, Hkv, G + 2, D), device=dev, dtype=torch.bfloat16)
     k_view, v_view = proj[..., -2, :], proj[..., -1, :]
-    ms_t = _time_fn(torch, lambda: ops.quantize_pack_token(v_view, bits), 10, 3)
+    ms_t = _time_fn(torch, lambda: ops.quantize_pack_token(v_view, bits), 40, 10)
     # per-token values: every buffer set gets values of its own, so the calls rotate over as many
     # distinct code buffers as the headline measurement does
     calls = []

@@ -34,6 +34,7 @@ struct QuantGeom {
     int64_t sb, st, sh;   // element strides of x
     int nchunk, chunk;    // token chunks
     FastDiv dT, dH;       // divisors T and H of a flat (b, h, t) row index (per-token quantiser)
+    FastDiv dTB;          // per-token quantiser: blocks of 16 tokens per (batch, head)
     int shared_stats;     // non-zero: one row of statistics / thresholds serves every (batch, head) (whole-tensor mode)
 };
 
@@ -973,26 +974,24 @@ __global__ __launch_bounds__(kQThreads) void token_pack_kernel(const uint16_t* _
                                                                uint16_t* __restrict__ scale,
                                                                uint16_t* __restrict__ mins) {
     constexpr float levels = static_cast<float>((1 << BITS) - 1);
-    const int64_t rows = static_cast<int64_t>(g.B) * g.H * g.T;
     const int l16 = threadIdx.x & 15, q4 = threadIdx.x & 3, grp = l16 >> 2;
     const float inv_levels = __fdiv_rn(1.0f, levels);
-    for (int64_t row = blockIdx.x * static_cast<int64_t>(kQThreads / 16) + (threadIdx.x >> 4); row < rows;
-         row += static_cast<int64_t>(gridDim.x) * (kQThreads / 16)) {
-        // output row order (b, h, t); row indices below 2^31 are split with host-prepared
-        // multipliers instead of 64-bit divisions
-        int t, h, b;
-        if (rows < (static_cast<int64_t>(1) << 31)) {
-            const uint32_t r32 = static_cast<uint32_t>(row);
-            const uint32_t bh = g.dT.quot(r32);
-            t = static_cast<int>(r32 - bh * g.dT.div);
-            const uint32_t bq = g.dH.quot(bh);
-            h = static_cast<int>(bh - bq * g.dH.div);
-            b = static_cast<int>(bq);
-        } else {
-            t = static_cast<int>(row % g.T);
-            h = static_cast<int>((row / g.T) % g.H);
-            b = static_cast<int>(row / (static_cast<int64_t>(g.T) * g.H));
-        }
+    // A workgroup pass is 16 consecutive tokens of one (batch, head).  Consecutive workgroups take the heads of the
+    // same 16 tokens, then the next 16 tokens: what is in flight on the device at any moment then covers whole token
+    // rows of x.  (Walking the output order (b, h, t) instead, everything in flight reads the same 256-byte column of
+    // its token rows - one head - and a contiguous (B, T, H, D) input then keeps a fraction of the memory channels
+    // busy.)
+    const uint32_t ntb = g.dTB.div;                                   // 16-token blocks per (batch, head)
+    const int64_t nblk = static_cast<int64_t>(g.B) * g.H * ntb;      // (the host keeps this below 2^31)
+    for (int64_t blk = blockIdx.x; blk < nblk; blk += gridDim.x) {
+        const uint32_t b32 = static_cast<uint32_t>(blk);
+        const uint32_t bt = g.dH.quot(b32);                           // (b, token block)
+        const int h = static_cast<int>(b32 - bt * g.dH.div);
+        const uint32_t bq = g.dTB.quot(bt);
+        const int b = static_cast<int>(bq);
+        const int t = static_cast<int>(bt - bq * ntb) * (kQThreads / 16) + static_cast<int>(threadIdx.x >> 4);
+        if (t >= g.T) continue;   // (the 16 lanes of a row leave together)
+        const int64_t row = (static_cast<int64_t>(b) * g.H + h) * g.T + t;   // output row order (b, h, t)
         const uint4 v = *reinterpret_cast<const uint4*>(x + b * g.sb + t * g.st + h * g.sh + l16 * 8);
         float f[8];
         unpack8<DT>(v, f);
@@ -1012,17 +1011,30 @@ __global__ __launch_bounds__(kQThreads) void token_pack_kernel(const uint16_t* _
         const float m1 = s * (0.5f + 0.001953125f);      // 0.5 + 2^-9
         const float m2 = s * (1.5f - 0.00390625f);       // 1.5 - 2^-8
         const float m3 = s * (2.5f + 0.0078125f);        // 2.5 + 2^-7
+        // ... and d = bf16(y), y = fp32(x - min) >= 0, is a monotone function of y, so each of those comparisons is
+        // one comparison of y itself: with u the smallest bf16 value that satisfies it (the one above m for ">", m
+        // rounded up for ">="), bf16(y) >= u exactly when y lies above the midpoint between u and the bf16 value
+        // below it, or on it if u is the even one of the two (round-half-even).  In the bit patterns of positive
+        // floats that midpoint is u - 0x8000, also across a power of two.  One subtraction and one comparison per
+        // element instead of a subtraction, a rounding and a comparison.
+        auto from = [](float m, bool inclusive) -> float {
+            const uint32_t mb = __float_as_uint(m);
+            const uint32_t ub = inclusive ? ((mb + 0xffffu) & 0xffff0000u) : ((mb & 0xffff0000u) + 0x10000u);
+            const uint32_t mid = ub - 0x8000u;
+            return __uint_as_float((ub & 0x10000u) ? mid + 1u : mid);
+        };
+        const float y1 = from(m1, false), y2 = from(m2, true), y3 = from(m3, false);
         uint32_t packed = 0;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const float d = rnd<DT>(f[i] - mn);
+            const float y = f[i] - mn;
             uint32_t code = 0;
             if (by_compare) {
-                code = (d > m1) ? 1u : 0u;
-                if constexpr (BITS == 2) code += ((d >= m2) ? 1u : 0u) + ((d > m3) ? 1u : 0u);
+                code = (y >= y1) ? 1u : 0u;
+                if constexpr (BITS == 2) code += ((y >= y2) ? 1u : 0u) + ((y >= y3) ? 1u : 0u);
             } else {
-                const float y = rnd<DT>(__fdiv_rn(d, s));
-                if (y == y) code = static_cast<uint32_t>(rintf(fminf(fmaxf(y, 0.0f), levels)));
+                const float q = rnd<DT>(__fdiv_rn(rnd<DT>(y), s));
+                if (q == q) code = static_cast<uint32_t>(rintf(fminf(fmaxf(q, 0.0f), levels)));
             }
             packed |= code << (BITS * i);
         }
@@ -1169,8 +1181,11 @@ int cq_quantize_pack_token(const void* x, int dtype, int B, int T, int H, int D,
     g.nchunk = 1; g.chunk = T;
     g.dT.set(static_cast<uint32_t>(T));
     g.dH.set(static_cast<uint32_t>(H));
-    const int64_t rows = static_cast<int64_t>(B) * H * T;
-    int64_t blocks = (rows + cq::kQThreads / 16 - 1) / (cq::kQThreads / 16);
+    const int64_t ntb = (static_cast<int64_t>(T) + cq::kQThreads / 16 - 1) / (cq::kQThreads / 16);
+    g.dTB.set(static_cast<uint32_t>(ntb));
+    const int64_t nblk = static_cast<int64_t>(B) * H * ntb;
+    if (nblk > 0x7fffffff) return CQ_ERR_SHAPE;
+    int64_t blocks = nblk;
     if (blocks > (1 << 20)) blocks = 1 << 20;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const uint16_t* xp = static_cast<const uint16_t*>(x);
