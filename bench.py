@@ -253,7 +253,7 @@ def side_legs(torch, ops, shape, bits, sets, settle_ms=0.0, only_token=False):
     del calls
     if only_token:
         return res
-    # the other bit width of the same layer shape (BASELINE's layer configuration names b = 1 and b = 2)
+    # the other bit width of the same layer shape (the benchmark's layer configuration names b = 1 and b = 2)
     ob = 2 if bits == 1 else 1
     osets = build_sets(torch, ops, shape, ob, 2 if ob == 2 else len(sets), 4321)
     ocalls = [ops.DecodeCall(x["q"], x["ck"], x["cv"], x["sk"], x["zk"], x["sv"], x["zv"], x["kr"], x["vr"],

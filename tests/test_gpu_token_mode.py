@@ -86,7 +86,7 @@ def test_decode_attn_token_values_split_path(bits):
 
 @pytest.mark.parametrize("bits", [1, 2])
 def test_token_quantiser_full_size_matches_the_torch_device_op_chain(bits):
-    """BASELINE layer shape (64 x 3328 x 8 x 128, bf16): the kernel's words / scales / minima equal what
+    """Benchmark layer shape (64 x 3328 x 8 x 128, bf16): the kernel's words / scales / minima equal what
     the reference's sequence of torch ops (qjl/new_pack.py:64-72) gives on this GPU, and the words
     unpack to codes in range that reach 0 and L in every group."""
     from calibquant_amd import ops
