@@ -627,6 +627,12 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                 }
             }
         };
+        // The min/max launch has no value rows, tables or sums to keep: with the logits in registers it also keeps
+        // the packed K rows of all its tokens there across the table passes instead of requesting, in every pass, the
+        // 16-byte piece that pass looks at (at 2 bits, four passes: 214 MB fetched for 67 MB of rows at batch 8 x
+        // 32 768 - the rows of the 512 workgroups in flight do not fit the L2s between two passes).
+        constexpr bool kKeepRows = MINMAX_ONLY && REGL > 0 && L::KPASS > 1;
+        uint4 kall[kKeepRows ? REGL : 1][BITS];
         auto k_pass = [&](auto pass_c) {
             constexpr int P = decltype(pass_c)::value;
             constexpr int kP0 = (P * L::WPP) / 4;   // first 16-byte piece of a row the pass looks at
@@ -659,7 +665,28 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
 #undef CQ_K_ROUND
             static_assert(L::KR <= 4, "rounds are written out up to 4");
             uint4 kx[L::KR][L::PCS];   // rows beyond the first batch: this pass's pieces only
-            if constexpr (REGL > 0) {
+            if constexpr (kKeepRows) {
+                // whole rows, requested in the first pass and kept for the later ones
+#pragma unroll
+                for (int ob = 1; ob < (REGL + L::KR - 1) / L::KR; ++ob) {
+                    const int tb = ob * kNT * L::KR;
+                    if (tb < n) {
+                        if constexpr (P == 0) {
+#pragma unroll
+                            for (int r = 0; r < L::KR; ++r) {
+                                const int tt = min(tb + tid + r * kNT, n - 1);
+#pragma unroll
+                                for (int i = 0; i < BITS; ++i)
+                                    if (ob * L::KR + r < REGL) kall[ob * L::KR + r][i] = ckp[static_cast<int64_t>(tt) * BITS + i];
+                            }
+                        }
+#pragma unroll
+                        for (int r = 0; r < L::KR; ++r)
+                            if (ob * L::KR + r < REGL)
+                                token_logits(pass_c, ob * L::KR + r, tb + tid + r * kNT, kall[ob * L::KR + r] + kP0);
+                    }
+                }
+            } else if constexpr (REGL > 0) {
                 // batches written out, so that the logits' registers are indexed by constants
 #pragma unroll
                 for (int ob = 1; ob < (REGL + L::KR - 1) / L::KR; ++ob) {
