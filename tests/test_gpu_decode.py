@@ -412,3 +412,39 @@ def test_decode_attn_chunked_with_the_logits_buffer(ops, case):
     out2 = call.run()
     torch.cuda.synchronize()
     assert torch.equal(out, out2)
+
+
+@pytest.mark.parametrize("case", [(1, 32, 8, 20000, 40, 3, 1), (8, 32, 8, 12000, 0, 0, 1), (2, 32, 8, 12000, 33, 0, 2)],
+                         ids=lambda c: "-".join(str(x) for x in c))
+def test_decode_attn_chunked_launches_replayed_from_a_graph(ops, case):
+    """The two chunked launches (counters cleared by the first, partials merged by the last workgroup of a unit in
+    the second; logits through the workspace or recomputed) recorded into a HIP graph: every replay, with eager
+    work and synchronisations in between, gives the bits of the eager call."""
+    B, Hq, Hkv, T, R, S, bits = case
+    c = make_case(1, Hq, Hkv, 128, T, max(R, 1), bits, "bf16", seed=700 + T + bits, outlier_kind="student")
+    g = {k: torch.cat([v] * B, 0) for k, v in case_to_gpu(c, "bf16").items()}
+    call = ops.DecodeCall(g["q"], g["ck"], g["cv"], g["sk"], g["zk"], g["sv"], g["zv"], g["kr"] if R else None,
+                          g["vr"] if R else None, sprompt_len=S, bits=bits)
+    assert call.plan()["chunks"] > 1
+    eager = call.run().clone()
+    torch.cuda.synchronize()
+    want = O.decode_attention(c["q"], c["ck"], c["cv"], c["sk"], c["zk"], c["sv"], c["zv"],
+                              c["kr"][:, :, :R] if R else None, c["vr"][:, :, :R] if R else None, S, bits)
+    _check(to_np(eager[:1]), want)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        call.run()                                   # warm-up on the capture stream
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            call.run()
+    for i in range(4):
+        call.out.zero_()
+        other = call.run().clone() if i == 2 else None       # an eager call between two replays
+        call.out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(call.out, eager), i
+        if other is not None:
+            assert torch.equal(other, eager)
