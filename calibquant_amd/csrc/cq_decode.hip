@@ -264,7 +264,10 @@ __device__ __forceinline__ uint32_t pack_f16(float a, float b) {
     return __builtin_bit_cast(uint32_t, h);
 }
 
-template <int BITS, int HPB, typename DT, bool MINMAX_ONLY, bool VTOK = false, int NT = 1024, int REGL = 0>
+// CHUNKED: the launch is one of the two of a chunked step (the min/max launch always is); a single launch carries
+// none of their code
+template <int BITS, int HPB, typename DT, bool MINMAX_ONLY, bool VTOK = false, int NT = 1024, int REGL = 0,
+          bool CHUNKED = MINMAX_ONLY>
 // (four waves per SIMD - at most 128 VGPRs - for either workgroup size: two 512-thread workgroups per compute
 // unit are only resident together within that)
 __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
@@ -326,7 +329,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
 
     const bool img_unit = split < g.nsplit && g.T > 0;
     const int R = g.r_dev ? min(*g.r_dev, g.R) : g.R;   // rows in the residual window
-    const bool do_res = !MINMAX_ONLY && R > 0 && (g.nsplit == 1 || split == g.nsplit);
+    const bool do_res = !MINMAX_ONLY && R > 0 && (!CHUNKED || split == g.nsplit);
     const int t0 = img_unit ? split * g.chunk : 0;
     const int n = img_unit ? min(g.T, t0 + g.chunk) - t0 : 0;
     const int npad = (n + L::TPW - 1) / L::TPW * L::TPW;
@@ -344,7 +347,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
     // launch takes them from there - no packed K rows, no table, no look-ups of its own
     const int64_t unit = bh * static_cast<int64_t>(g.d_ng.div) + hg;
     V* gl = reinterpret_cast<V*>(g.lgt) + (unit * g.T + t0);
-    const bool from_gl = !MINMAX_ONLY && g.lgt != nullptr && has_img;
+    const bool from_gl = !MINMAX_ONLY && CHUNKED && g.lgt != nullptr && has_img;
     const bool k_rows = has_img && !from_gl;
     uint32_t q_raw, s_raw, z_raw;
     constexpr bool kVSep = (HPB * kD > kNT - kD);
@@ -447,7 +450,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
     // REGL: the logits of this thread's tokens, round r = token tid + r * kNT
     V lg[REGL > 0 ? REGL : 1];
     if constexpr (!MINMAX_ONLY) {
-        if (g.nsplit > 1 && has_img) {
+        if (CHUNKED && has_img) {
 #pragma unroll
             for (int h = 0; h < HPB; ++h) {
                 const MinMax* p = reinterpret_cast<const MinMax*>(g.mm) +
@@ -793,7 +796,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             }
 
             // ---- phase 4: calibration + exp ---------------------------------------------
-            if (g.nsplit > 1) {   // one fold for both: max of (-min, max) over the chunks
+            if constexpr (CHUNKED) {   // one fold for both: max of (-min, max) over the chunks
                 float mm2[2 * HPB];
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) {
@@ -1213,7 +1216,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             const float mr = stat[HPB + h], lr = stat[2 * HPB + h];
             const float mi = stat[3 * HPB + h], li = stat[4 * HPB + h];
             const int64_t row = static_cast<int64_t>(b) * g.Hq + hq0 + h;
-            if (g.nsplit == 1) {
+            if constexpr (!CHUNKED) {
                 const float mf = fmaxf(mi, mr);
                 const float wi = (mi == -INFINITY) ? 0.f : __expf(mi - mf);
                 const float wr = (mr == -INFINITY) ? 0.f : __expf(mr - mf);
@@ -1227,7 +1230,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                 publish(p + 2 + d, is_img ? o_img : o_res);
             }
         }
-        if (g.nsplit > 1) {
+        if constexpr (CHUNKED) {
             // The unit's chunks (and its residual unit) each leave an (m, l, acc) partial; the workgroup that
             // finds all the others' already counted combines them.  The partials are device-scope atomic stores
             // (written through to the level all compute units share, so no cache has to be written back as a
@@ -1430,7 +1433,8 @@ template <int BITS, int HPB, typename DT, bool VTOK, int NT = 1024, int REGL = 0
 static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
     const int G = g.Hq / g.Hkv;
     const unsigned units = static_cast<unsigned>(g.B) * g.Hkv * ngroups(G, HPB);
-    auto kmain = decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL>;
+    auto kmain = g.nsplit > 1 ? decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, true>
+                              : decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, false>;
     auto kmm = decode_kernel<BITS, HPB, DT, true, false, NT, REGL>;   // the min/max pass never looks at values
     // raise the dynamic-LDS limit once per device for this instantiation
     static std::atomic<uint32_t> attr_done{0};
@@ -1439,15 +1443,15 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
     const uint32_t bit = 1u << (dev & 31);
     if (!(attr_done.load(std::memory_order_acquire) & bit)) {
         // the K look-ups address the table absolutely: the dynamic LDS array must start at 0
-        hipFuncAttributes fa;
-        CQ_HIP_CHECK(hipFuncGetAttributes(&fa, reinterpret_cast<const void*>(kmain)));
-        if (fa.sharedSizeBytes != 0) return CQ_ERR_LAUNCH;
-        CQ_HIP_CHECK(hipFuncGetAttributes(&fa, reinterpret_cast<const void*>(kmm)));
-        if (fa.sharedSizeBytes != 0) return CQ_ERR_LAUNCH;
-        CQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kmain),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax));
-        CQ_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kmm),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax));
+        const void* kernels[3] = {reinterpret_cast<const void*>(decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, false>),
+                                  reinterpret_cast<const void*>(decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, true>),
+                                  reinterpret_cast<const void*>(kmm)};
+        for (const void* k : kernels) {
+            hipFuncAttributes fa;
+            CQ_HIP_CHECK(hipFuncGetAttributes(&fa, k));
+            if (fa.sharedSizeBytes != 0) return CQ_ERR_LAUNCH;
+            CQ_HIP_CHECK(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax));
+        }
         attr_done.fetch_or(bit, std::memory_order_release);
     }
     DecodeGeom gm = g;
