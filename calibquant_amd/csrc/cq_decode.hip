@@ -265,9 +265,11 @@ __device__ __forceinline__ uint32_t pack_f16(float a, float b) {
 }
 
 // CHUNKED: the launch is one of the two of a chunked step (the min/max launch always is); a single launch carries
-// none of their code
+// none of their code.  EXTRAS: an additive mask or a residual row count read from device memory may be present; a
+// call with neither runs an instantiation without their code (32.6-32.8 against 33.5-34.0 us at the benchmark shape:
+// the kernel sits at the register limit of its occupancy, and code that never runs still costs registers).
 template <int BITS, int HPB, typename DT, bool MINMAX_ONLY, bool VTOK = false, int NT = 1024, int REGL = 0,
-          bool CHUNKED = MINMAX_ONLY>
+          bool CHUNKED = MINMAX_ONLY, bool EXTRAS = !MINMAX_ONLY>
 // (four waves per SIMD - at most 128 VGPRs - for either workgroup size: two 512-thread workgroups per compute
 // unit are only resident together within that)
 __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
@@ -328,7 +330,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
     const int64_t bh = static_cast<int64_t>(b) * g.Hkv + hkv;
 
     const bool img_unit = split < g.nsplit && g.T > 0;
-    const int R = g.r_dev ? min(*g.r_dev, g.R) : g.R;   // rows in the residual window
+    const int R = (EXTRAS && g.r_dev) ? min(*g.r_dev, g.R) : g.R;   // rows in the residual window
     const bool do_res = !MINMAX_ONLY && R > 0 && (!CHUNKED || split == g.nsplit);
     const int t0 = img_unit ? split * g.chunk : 0;
     const int n = img_unit ? min(g.T, t0 + g.chunk) - t0 : 0;
@@ -826,7 +828,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                     slope[h] = 1.0f;
                 }
             }
-            if (g.mask) {
+            if (EXTRAS && g.mask) {
                 const float* mk = g.mask + b * g.mask_sb + g.S + t0;
                 float lm[HPB];
 #pragma unroll
@@ -1115,7 +1117,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             for (int k = 0; k < 2; ++k)
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) accv[k][h] = 0.f;
-            const float* mk = g.mask ? g.mask + b * g.mask_sb : nullptr;
+            const float* mk = (EXTRAS && g.mask) ? g.mask + b * g.mask_sb : nullptr;
 
             for (int r0 = 0; r0 < R; r0 += kResTile) {
                 const bool more = r0 + kResTile < R;
@@ -1433,8 +1435,11 @@ template <int BITS, int HPB, typename DT, bool VTOK, int NT = 1024, int REGL = 0
 static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
     const int G = g.Hq / g.Hkv;
     const unsigned units = static_cast<unsigned>(g.B) * g.Hkv * ngroups(G, HPB);
-    auto kmain = g.nsplit > 1 ? decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, true>
-                              : decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, false>;
+    const bool extras = g.mask != nullptr || g.r_dev != nullptr;
+    auto kmain = g.nsplit > 1 ? (extras ? decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, true, true>
+                                        : decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, true, false>)
+                              : (extras ? decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, false, true>
+                                        : decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, false, false>);
     auto kmm = decode_kernel<BITS, HPB, DT, true, false, NT, REGL>;   // the min/max pass never looks at values
     // raise the dynamic-LDS limit once per device for this instantiation
     static std::atomic<uint32_t> attr_done{0};
@@ -1443,8 +1448,10 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
     const uint32_t bit = 1u << (dev & 31);
     if (!(attr_done.load(std::memory_order_acquire) & bit)) {
         // the K look-ups address the table absolutely: the dynamic LDS array must start at 0
-        const void* kernels[3] = {reinterpret_cast<const void*>(decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, false>),
-                                  reinterpret_cast<const void*>(decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, true>),
+        const void* kernels[5] = {reinterpret_cast<const void*>(decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, false, false>),
+                                  reinterpret_cast<const void*>(decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, false, true>),
+                                  reinterpret_cast<const void*>(decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, true, false>),
+                                  reinterpret_cast<const void*>(decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, true, true>),
                                   reinterpret_cast<const void*>(kmm)};
         for (const void* k : kernels) {
             hipFuncAttributes fa;
