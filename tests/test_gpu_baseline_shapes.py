@@ -187,3 +187,24 @@ def test_full_8b_shaped_model_batch_64_first_and_last_layer_and_recorded_step():
         assert torch.equal(runs[0], runs[1])
     finally:
         InternLM2Attention.forward, InternVLChatStandIn.generate = fp_forward, fp_generate
+
+
+@pytest.mark.parametrize("bits", [1, 2])
+def test_long_context_chunked_step_is_deterministic_back_to_back(ops, bits):
+    """Sixty chunked steps queued back to back on one stream (the unit counters are cleared by each step's first
+    launch, the partials merged by whichever workgroup of a unit finishes last): every output equals the first,
+    which is checked against the oracle."""
+    c = make_case(1, 32, 8, 128, 32768, 16, bits, "bf16", seed=330 + bits, outlier_kind="student")
+    g = {k: torch.cat([v] * 8, 0) for k, v in case_to_gpu(c, "bf16").items()}
+    outs = [torch.empty((8, 32, 128), dtype=torch.bfloat16, device="cuda") for _ in range(60)]
+    call = ops.DecodeCall(g["q"], g["ck"], g["cv"], g["sk"], g["zk"], g["sv"], g["zv"], g["kr"], g["vr"],
+                          sprompt_len=3, bits=bits, out=outs[0])
+    assert call.plan()["chunks"] > 1
+    for o in outs:
+        call.args.out = o.data_ptr()
+        call.run()
+    torch.cuda.synchronize()
+    want = O.decode_attention(c["q"], c["ck"], c["cv"], c["sk"], c["zk"], c["sv"], c["zv"], c["kr"], c["vr"], 3, bits)
+    _check(to_np(outs[0][:1]), want, "first of sixty")
+    for i, o in enumerate(outs[1:]):
+        assert torch.equal(o, outs[0]), i + 1
