@@ -18,6 +18,10 @@ Before the W warm-up steps the same calls run untimed for `--settle-ms`
 steady state (a run of 20 steps straight after the inputs are built reads
 about 10 % slower than one of 4 000), and the steady state is what a decode
 loop of thousands of layer calls per second sees.  `config.settle_ms` states it.
+The timed block of K steps is repeated `--blocks` times (default 25) and the
+median block is `value` / `ms_per_step` (`config.timed_blocks`); the figure of a
+cold process - W warm-up steps and one block of K steps with no settling run -
+is reported beside it as `value_unsettled_us`.
 """
 from __future__ import annotations
 
@@ -107,10 +111,8 @@ def settle(torch, run, ms):
     torch.cuda.synchronize()
 
 
-def time_calls(torch, calls, steps, warmup, settle_ms=0.0):
-    settle(torch, lambda i: calls[i % len(calls)].run(), settle_ms)
-    for i in range(warmup):
-        calls[i % len(calls)].run()
+def time_block(torch, calls, steps):
+    """One timed block: exactly `steps` calls between two events, synchronised on both sides; ms per call."""
     torch.cuda.synchronize()
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
@@ -118,7 +120,18 @@ def time_calls(torch, calls, steps, warmup, settle_ms=0.0):
         calls[i % len(calls)].run()
     end.record()
     torch.cuda.synchronize()
-    return start.elapsed_time(end) / steps  # ms per call
+    return start.elapsed_time(end) / steps
+
+
+def time_calls(torch, calls, steps, warmup, settle_ms=0.0, blocks=1):
+    """`warmup` untimed calls, then `blocks` timed blocks of exactly `steps` calls each; the median block
+    is the figure (a single block of 20 calls lasts under a millisecond and reads a few per cent high or
+    low from one run to the next).  Returns (median ms per call, [every block's ms per call])."""
+    settle(torch, lambda i: calls[i % len(calls)].run(), settle_ms)
+    for i in range(warmup):
+        calls[i % len(calls)].run()
+    per = sorted(time_block(torch, calls, steps) for _ in range(max(1, blocks)))
+    return per[len(per) // 2], per
 
 
 def time_fp16_kv(torch, shape, steps, warmup, nsets):
@@ -244,7 +257,7 @@ def side_legs(torch, ops, shape, bits, sets, settle_ms=0.0, only_token=False):
         calls.append(ops.DecodeCall(x["q"], x["ck"], words, x["sk"], x["zk"], vsc, vmn, x["kr"], x["vr"],
                                     sprompt_len=S, bits=bits, v_mode="token"))
     del proj, k_view, v_view
-    ms_d = time_calls(torch, calls, 200, 20, settle_ms)
+    ms_d, _ = time_calls(torch, calls, 200, 20, settle_ms, 5)
     nb = algorithmic_bytes(B, Hq, Hkv, D, T, R, bits) - 2 * B * Hkv * D * 2 + 2 * B * Hkv * T * (D // 32) * 2
     res["per_token_values"] = {"quantize_pack_token_us": round(ms_t * 1e3, 1), "decode_us_layer": round(ms_d * 1e3, 2),
                                "algorithmic_bytes": nb, "achieved_GBps": round(nb / ms_d / 1e6, 1),
@@ -258,7 +271,7 @@ def side_legs(torch, ops, shape, bits, sets, settle_ms=0.0, only_token=False):
     osets = build_sets(torch, ops, shape, ob, 2 if ob == 2 else len(sets), 4321)
     ocalls = [ops.DecodeCall(x["q"], x["ck"], x["cv"], x["sk"], x["zk"], x["sv"], x["zv"], x["kr"], x["vr"],
                              sprompt_len=S, bits=ob) for x in osets]
-    ms_o = time_calls(torch, ocalls, 200, 20, settle_ms)
+    ms_o, _ = time_calls(torch, ocalls, 200, 20, settle_ms, 5)
     nbo = algorithmic_bytes(B, Hq, Hkv, D, T, R, ob)
     res[f"decode_{ob}bit"] = {"us_layer": round(ms_o * 1e3, 2), "algorithmic_bytes": nbo,
                               "achieved_GBps": round(nbo / ms_o / 1e6, 1),
@@ -474,6 +487,8 @@ def main():
                     help="also launch three 256 MiB device copies (known traffic, for scaling profiler byte counters)")
     ap.add_argument("--settle-ms", type=float, default=300.0,
                     help="untimed run of the same calls before the warm-up steps, in ms of device time")
+    ap.add_argument("--blocks", type=int, default=25,
+                    help="timed blocks of --steps calls each; the median block is reported")
     ap.add_argument("--only", default=None, choices=("prefill", "prefill-contiguous", "token-values"),
                     help="run one side figure alone (for profiling it) and print its JSON")
     ap.add_argument("--seed", type=int, default=1234)
@@ -507,7 +522,10 @@ def main():
         return
     calls = [ops.DecodeCall(s["q"], s["ck"], s["cv"], s["sk"], s["zk"], s["sv"], s["zv"], s["kr"], s["vr"],
                             sprompt_len=S, bits=a.bits) for s in sets]
-    ms = time_calls(torch, calls, a.steps, a.warmup, a.settle_ms)
+    # the same K steps after W warm-up calls straight after the inputs were built (no settling run, one
+    # block): the protocol of a cold process, reported next to the steady-state figure
+    ms_cold, _ = time_calls(torch, calls, a.steps, a.warmup, 0.0, 1)
+    ms, per_block = time_calls(torch, calls, a.steps, a.warmup, a.settle_ms, a.blocks)
     plan = calls[0].plan()
     nbytes = algorithmic_bytes(B, Hq, Hkv, D, T, R, a.bits)
     gbps = nbytes / (ms * 1e-3) / 1e9
@@ -527,10 +545,16 @@ def main():
         "data": "synthetic",
         "config": {"workload": a.workload, "batch": B, "q_heads": Hq, "kv_heads": Hkv, "head_dim": D,
                    "kv_packed_tokens": T, "kv_residual_rows": R, "bits": a.bits, "storage_dtype": "bf16",
-                   "buffer_sets": a.sets, "settle_ms": a.settle_ms, "launches_per_step": plan["launches"],
-                   "launch_plan": plan},
+                   "buffer_sets": a.sets, "settle_ms": a.settle_ms, "timed_blocks": a.blocks,
+                   "timing": f"median of {a.blocks} timed blocks of {a.steps} steps each, after {a.settle_ms:g} ms of "
+                             f"the same calls untimed and {a.warmup} warm-up steps",
+                   "launches_per_step": plan["launches"], "launch_plan": plan},
+        "value_unsettled_us": round(ms_cold * 1e3, 3),
+        "value_blocks_us": {"min": round(per_block[0] * 1e3, 3), "max": round(per_block[-1] * 1e3, 3)},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": measured_traffic(a.workload, a.bits),
+                     "traffic_source": "profiles/decode_kernel_traffic.json (rocprofv3 FETCH_SIZE / WRITE_SIZE of an "
+                                       "earlier run of this workload, scaled by a 256 MiB copy; not measured by this run)",
                      "algorithmic_bytes": nbytes},
     }
     if not a.no_fp16kv:

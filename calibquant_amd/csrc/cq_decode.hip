@@ -37,6 +37,13 @@
 // Everything here is HBM / LDS / VALU work; no matrix-core instructions.
 #include "cq_common.h"
 
+// The kernels below lean on behaviour of this architecture family that the HIP memory model does not
+// promise (see the in-launch merge of the chunked step) and on its LDS size, DPP controls and
+// instruction set: refuse to build device code for anything else.
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__) && !defined(__gfx942__)
+#error "cq_decode.hip is written for gfx950 (validated on gfx950 only; gfx942 shares the memory behaviour relied on)"
+#endif
+
 #include <atomic>
 #include <type_traits>
 
@@ -50,6 +57,24 @@ constexpr int kRegPair = 8;        // rounds of logits a thread of a 512-thread 
 constexpr int kRegTwoBit = 4;      // ... of the 2-bit kernel with four heads per unit (4 096 tokens)
 constexpr int kRegLong = 10;       // ... of a 1024-thread workgroup that holds a long chunk in one launch (10 240 tokens)
 constexpr float kLog2e = 1.4426950408889634f;
+#ifndef CQ_X_ROT
+#define CQ_X_ROT 1
+#endif
+#ifndef CQ_X_VPF
+#define CQ_X_VPF 1
+#endif
+#ifndef CQ_X_RES
+#define CQ_X_RES 0
+#endif
+#ifndef CQ_X_VREQ
+#define CQ_X_VREQ -1
+#endif
+#ifndef CQ_X_PRIO
+#define CQ_X_PRIO 1
+#endif
+#ifndef CQ_X_KENTRY
+#define CQ_X_KENTRY 0
+#endif
 
 template <int N> struct alignas(N * 4) Vec { float v[N]; };
 // native 16-byte vector: copies are single vector moves (HIP's uint4 struct copies lower to memcpy)
@@ -117,7 +142,13 @@ template <int BITS, int HPB, bool VTOK = false, int NT_ = 1024, int REGL = 0> st
     // table's share of the LDS (64 KB; 32 KB for a 512-thread workgroup), else half of them in each of
     // two (or a quarter in each of four) passes over the chunk's rows, the earlier passes' partial logits
     // waiting in the token slots or, with REGL, in registers.
-    static constexpr int KTMAX = (NT_ == 512 ? 32 : 64) * 1024;
+    // INA (512-thread workgroup with the logits in registers): nothing else lives in LDS while the K table is
+    // in use, so the table takes all 64 KB of region A and the token slots, written only after the last
+    // look-up, sit in that region as well, behind the staged V block - one table pass at 1 bit (two at 2 bits)
+    // with 256-byte rows, i.e. single-permute look-up addresses, inside the 80 KB a paired workgroup may use.
+    // The table is then built straight from the per-bit weights (no nibble tables to find room for).
+    static constexpr bool INA = (NT_ == 512 && REGL > 0);
+    static constexpr int KTMAX = ((NT_ == 512 && !INA) ? 32 : 64) * 1024;
     static constexpr int KPASS = (NB * 256 * ESZ > 2 * KTMAX) ? 4 : (NB * 256 * ESZ > KTMAX) ? 2 : 1;
     static constexpr int NBP = NB / KPASS;          // byte positions per pass
     static constexpr int WPP = NBP / 4;             // 32-bit words of a row per pass
@@ -141,16 +172,21 @@ template <int BITS, int HPB, bool VTOK = false, int NT_ = 1024, int REGL = 0> st
     static constexpr int F_STAT = F_RED + kNW * RW;           // 8*HPB: per-head softmax state
     static constexpr int F_VSZ = F_STAT + 8 * HPB;            // 2*kD: value scale, zero-point (VTOK: NGRP*HPB minimum terms)
     static constexpr int F_NIB = F_VSZ + 2 * kD;              // NB*32*HPB: nibble tables
-    // (REGL: the nibble tables live in the token slots, which are first written after the last table pass)
+    // (REGL: the nibble tables live in the token slots, which are first written after the last table pass;
+    // INA: there are none)
     static constexpr int NIBF = NB * 32 * HPB;
     static constexpr int F_SRES = F_NIB + (REGL > 0 ? 0 : NIBF);  // kResTile*HPB
     static constexpr int F_PRES = F_SRES + kResTile * HPB;    // kResTile*HPB
     static constexpr int F_END = F_PRES + kResTile * HPB;
     static constexpr int FIXED = ((F_END * 4 + 255) / 256) * 256;
+    // byte offset of the token slots: behind the fixed region, or (INA) inside region A behind the staged V block
+    static constexpr int slots_in_a(int cap) { return WTAB + cmin(VSUB, cap) * NB; }
     static constexpr int region_a(int cap) {
-        return (cmax(cmax(KT, WTAB + cmin(VSUB, cap) * NB), cmax(RED, RED2)) + 255) / 256 * 256;
+        return (cmax(cmax(KT, slots_in_a(cap) + (INA ? cap * SLOT : 0)), cmax(RED, RED2)) + 255) / 256 * 256;
     }
-    static constexpr int lds_bytes(int cap) { return region_a(cap) + FIXED + cmax(cap * SLOT, REGL > 0 ? NIBF * 4 : 0); }
+    static constexpr int lds_bytes(int cap) {
+        return region_a(cap) + FIXED + (INA ? 0 : cmax(cap * SLOT, REGL > 0 ? NIBF * 4 : 0));
+    }
     // largest chunk whose layout fits: the whole LDS for a 1024-thread workgroup, half of it for a
     // 512-thread workgroup (two are meant to be resident per compute unit)
     static constexpr int max_chunk() {
@@ -281,7 +317,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
     const int reg_a = L::region_a(g.cap);
     unsigned char* regA = smem;
     float* fx = reinterpret_cast<float*>(smem + reg_a);
-    unsigned char* slots = smem + reg_a + L::FIXED;   // one slot per token of the chunk
+    unsigned char* slots = L::INA ? smem + L::slots_in_a(g.cap) : smem + reg_a + L::FIXED;   // one slot per token of the chunk
     auto slot = [&](int t) { return slots + t * L::SLOT; };
     float* wbit = fx + L::F_WBIT;
     float* qsz = fx + L::F_QSZ;
@@ -308,10 +344,23 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
         constexpr int PH = decltype(phase_c)::value;   // 0 set-up and tables, 1 K look-ups, 2 min/max .. exp, 3 packed V, 4 folds, window, merge
         if constexpr (NT == 512) {
             if (prio_on) {
+#if CQ_X_PRIO == 1
                 if constexpr (PH == 0 || PH == 2) __builtin_amdgcn_s_setprio(2);
                 else if constexpr (PH == 1) { if (second) __builtin_amdgcn_s_setprio(0); else __builtin_amdgcn_s_setprio(1); }
                 else if constexpr (PH == 3) { if (second) __builtin_amdgcn_s_setprio(2); else __builtin_amdgcn_s_setprio(1); }
                 else __builtin_amdgcn_s_setprio(0);
+#elif CQ_X_PRIO == 2   // latency phases above the loops, loops equal
+                if constexpr (PH == 0 || PH == 2) __builtin_amdgcn_s_setprio(2);
+                else if constexpr (PH == 1 || PH == 3) __builtin_amdgcn_s_setprio(1);
+                else __builtin_amdgcn_s_setprio(2);
+#elif CQ_X_PRIO == 3   // as 1, tail phases high
+                if constexpr (PH == 0 || PH == 2) __builtin_amdgcn_s_setprio(2);
+                else if constexpr (PH == 1) { if (second) __builtin_amdgcn_s_setprio(0); else __builtin_amdgcn_s_setprio(1); }
+                else if constexpr (PH == 3) { if (second) __builtin_amdgcn_s_setprio(2); else __builtin_amdgcn_s_setprio(1); }
+                else __builtin_amdgcn_s_setprio(3);
+#elif CQ_X_PRIO == 4   // first workgroup ahead everywhere
+                if (second) __builtin_amdgcn_s_setprio(0); else __builtin_amdgcn_s_setprio(1);
+#endif
             }
         }
     };
@@ -376,6 +425,15 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
     const U4* cvp4 = reinterpret_cast<const U4*>(cvp);
     const int last_u = has_img ? n * NB / 16 - 1 : 0;   // last valid 16-byte unit of either stream
     const int last_uk = k_rows ? last_u : 0;
+    uint4 kc[L::KR][BITS];
+    constexpr bool kKEntry = CQ_X_KENTRY && L::INA;
+    if constexpr (kKEntry) {
+#pragma unroll
+        for (int r = 0; r < L::KR; ++r) {
+#pragma unroll
+            for (int i = 0; i < BITS; ++i) kc[r][i] = ckp[min((tid + r * kNT) * BITS + i, last_uk)];
+        }
+    }
     // residual tile: K slice (row = tid / LPR, 128 / LPR elements); V: a wave owns RPW rows of the tile and a
     // lane one channel pair of each of them, so the value products need no fold inside the wave
     constexpr int LPR = L::LPR, NKP = L::NKP, RPW = L::RPW;
@@ -438,11 +496,12 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
     // The packed K rows are requested only now: a wave that has to queue 64 KB of requests
     // first gets to phase 0 thousands of cycles later, and the table build below covers
     // their latency anyway.
-    uint4 kc[L::KR][BITS];
+    if constexpr (!kKEntry) {
 #pragma unroll
-    for (int r = 0; r < L::KR; ++r) {
+        for (int r = 0; r < L::KR; ++r) {
 #pragma unroll
-        for (int i = 0; i < BITS; ++i) kc[r][i] = ckp[min((tid + r * kNT) * BITS + i, last_uk)];
+            for (int i = 0; i < BITS; ++i) kc[r][i] = ckp[min((tid + r * kNT) * BITS + i, last_uk)];
+        }
     }
     // Chunked launch: the chunks' logit min / max, lane s the pair of chunk s for every head (all in flight
     // together; they are folded across the wave where the calibration needs them), and - with a logits
@@ -500,7 +559,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
     // rest as the K registers free up, so it has arrived when the logits are done.
     U4 vc[kPF];
     auto request_v = [&](int r) { vc[r] = cvp4[min((tid + (r / BITS) * kNT) * BITS + r % BITS, last_u)]; };
-    constexpr int kVEarly = kPF / 2;
+    constexpr int kVEarly = (CQ_X_VREQ >= 0 && L::INA && L::KPASS == 1) ? 0 : kPF / 2;
     if constexpr (!MINMAX_ONLY) {
 #pragma unroll
         for (int r = 0; r < kVEarly; ++r) request_v(r);
@@ -518,6 +577,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
         // zero-point sum of the byte position is folded into the high half.
         V* nib = REGL > 0 ? reinterpret_cast<V*>(slots) : reinterpret_cast<V*>(fx + L::F_NIB);   // [half*16 + value][byte position]
         V* ktab = reinterpret_cast<V*>(regA);           // [byte value][byte position]
+        if constexpr (!L::INA)
         for (int e = tid; e < NB * 32; e += kNT) {
             const int j = e % NB, half = (e / NB) >> 4, v = (e / NB) & 15;
             // position-fastest: the lanes of a wave read consecutive entries
@@ -535,7 +595,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             }
             nib[e] = acc;
         }
-        __syncthreads();
+        if constexpr (!L::INA) __syncthreads();
 
         phase_priority(std::integral_constant<int, 1>{});
         // ---- phase 3: logits of the chunk ------------------------------------------------
@@ -641,6 +701,44 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
         auto k_pass = [&](auto pass_c) {
             constexpr int P = decltype(pass_c)::value;
             constexpr int kP0 = (P * L::WPP) / 4;   // first 16-byte piece of a row the pass looks at
+            if constexpr (L::INA) {
+                // Straight from the per-bit weights: a thread owns (position, high nibble, bit 3) and writes the
+                // eight entries of the low three bits - the part common to all eight first, then one or two adds
+                // per entry; a wave writes four whole 256-byte rows at a time.
+                static_assert(!L::INA || (NBP == 16 && kNT == 512), "thread mapping of the direct table build");
+                const int pos = tid & 15, hv = (tid >> 4) & 15, b3 = tid >> 8;
+                const V* wb = reinterpret_cast<const V*>(wbit) + P * NBP + pos;
+                const V zs = reinterpret_cast<const V*>(qsz)[P * NBP + pos];
+                V base;
+#pragma unroll
+                for (int h = 0; h < HPB; ++h) base.v[h] = -zs.v[h];
+#pragma unroll
+                for (int bt = 3; bt < 8; ++bt) {
+                    const V w4 = wb[bt * NB];
+                    const float f = static_cast<float>(bt == 3 ? b3 : (hv >> (bt - 4)) & 1);
+#pragma unroll
+                    for (int h = 0; h < HPB; ++h) base.v[h] += f * w4.v[h];
+                }
+                const V w0 = wb[0], w1 = wb[NB], w2 = wb[2 * NB];
+                V hp[2], p01;
+#pragma unroll
+                for (int h = 0; h < HPB; ++h) {
+                    hp[0].v[h] = base.v[h];
+                    hp[1].v[h] = base.v[h] + w2.v[h];
+                    p01.v[h] = w0.v[h] + w1.v[h];
+                }
+                V* row = ktab + (hv * 16 + b3 * 8) * NBP + pos;
+#pragma unroll
+                for (int l = 0; l < 8; ++l) {
+                    V o = hp[l >> 2];
+                    if ((l & 3) != 0) {
+                        const V& ad = (l & 3) == 1 ? w0 : (l & 3) == 2 ? w1 : p01;
+#pragma unroll
+                        for (int h = 0; h < HPB; ++h) o.v[h] += ad.v[h];
+                    }
+                    row[l * NBP] = o;
+                }
+            } else {
             // byte table of the pass's positions = high-nibble table + low-nibble table
             for (int e = tid; e < NBP * 256; e += kNT) {
                 const int j = P * NBP + e % NBP, v = e / NBP;
@@ -651,7 +749,25 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                 for (int h = 0; h < HPB; ++h) o.v[h] = hi.v[h] + lo.v[h];
                 ktab[e] = o;
             }
+            }
             __syncthreads();
+            // One table pass, logits in registers: the rows stream through the KR row registers - when a
+            // round's row has been looked up its registers take the row of KR rounds later, so KR rounds
+            // are in flight while one is worked on and no batch of rows is waited for as a whole.
+            constexpr bool kRotate = CQ_X_ROT && L::KPASS == 1 && REGL > 0;
+            if constexpr (kRotate) {
+                static_assert(!kRotate || BITS == 1, "one 16-byte piece per row");
+#pragma unroll
+                for (int rd = 0; rd < REGL; ++rd) {
+                    token_logits(pass_c, rd, tid + rd * kNT, kc[rd % L::KR]);
+                    if (rd + L::KR < REGL) kc[rd % L::KR][0] = ckp[min(tid + (rd + L::KR) * kNT, last_uk)];
+                    if constexpr (!MINMAX_ONLY) {
+                        if constexpr (CQ_X_VREQ >= 0) { if (rd >= CQ_X_VREQ && rd < CQ_X_VREQ + kPF) request_v(rd - CQ_X_VREQ); }
+                        else if (rd < kPF - kVEarly) request_v(kVEarly + rd);   // the rest of the first packed V block
+                    }
+                }
+                return;
+            }
             // first batch: rows already in registers; each consumed round of the last pass frees
             // registers that take the first block of packed V rows
             // (written out round by round with constant indices so vc stays in registers)
@@ -796,6 +912,17 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                     stage_piece(vc[r], tok, r % BITS, tok < vn0);
                 }
             }
+            // The registers of the staged block take the next block's rows right away (clamped addresses when
+            // there is none), and the first residual tile is requested behind them: everything the rest of the
+            // unit reads is in flight while the exponentials and the packed-V loop run, instead of each stream
+            // being asked for when its phase starts - all workgroups of a launch reach their phases together, and
+            // the memory system would idle through the vector-bound phases and then see every request at once.
+            constexpr bool kVAhead = CQ_X_VPF && L::INA;
+            constexpr int kResAhead = L::INA ? CQ_X_RES : 0;
+            auto request_v_block = [&](int vs0) {
+#pragma unroll
+                for (int r = 0; r < kPF; ++r) vc[r] = cvp4[min((vs0 + tid + (r / BITS) * kNT) * BITS + r % BITS, last_u)];
+            };
 
             // ---- phase 4: calibration + exp ---------------------------------------------
             if constexpr (CHUNKED) {   // one fold for both: max of (-min, max) over the chunks
@@ -903,6 +1030,10 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             // keeps its partial through the packed-V phase and the fold rides on that phase's
             // closing barriers.
             __syncthreads();   // publishes e and vst
+            // (requested here, not right after the staging: the logits' registers are free now)
+            if constexpr (kVAhead) request_v_block(L::VSUB);
+            if constexpr (kResAhead >= 1) load_res_k(0, rk);
+            if constexpr (kResAhead >= 2) load_res_v(0, rv);
 
             // ---- phase 5: packed V ----------------------------------------------------------
             // lane = (byte column j, slice c of its 8 bit lanes); a wave pass covers TPW tokens
@@ -949,12 +1080,13 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                 const int vn = min(L::VSUB, npad - vs0);
                 if (vs0 > 0) {
                     __syncthreads();  // previous block consumed
+                    if constexpr (!kVAhead) request_v_block(vs0);
 #pragma unroll
                     for (int r = 0; r < kPF; ++r) {
                         const int tok = tid + (r / BITS) * kNT;
-                        const U4 c = cvp4[min((vs0 + tok) * BITS + r % BITS, last_u)];
-                        stage_piece(c, tok, r % BITS, tok < vn);
+                        stage_piece(vc[r], tok, r % BITS, tok < vn);
                     }
+                    if constexpr (kVAhead) request_v_block(vs0 + L::VSUB);
                     __syncthreads();
                 }
                 for (int u = wvu; u * L::TPW < vn; u += kNW) {   // wave-uniform loop control
@@ -1035,7 +1167,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                 }
             }
             phase_priority(std::integral_constant<int, 4>{});
-            load_res_k(0, rk);   // first residual tile's K rows: in flight during the fold below
+            if constexpr (kResAhead < 1) load_res_k(0, rk);   // first residual tile's K rows: in flight during the fold below
             // per-wave partial sums of e (and of e * minimum), folded by the output threads below
             constexpr int kSums = VTOK ? (L::NGRP + 1) * HPB : HPB;
             wave_reduce_n<HPB>(ls, OpSum(), 0.f);
@@ -1096,7 +1228,11 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             __syncthreads();
         }
 
-        if (n == 0) load_res_k(0, rk);
+        constexpr int kResAhead2 = L::INA ? CQ_X_RES : 0;
+        if (n == 0) {
+            load_res_k(0, rk);
+            if constexpr (kResAhead2 >= 2) load_res_v(0, rv);
+        }
         // ---- phase 6: full-precision residual rows, online softmax.  Runs last: its first
         // tile is requested when the packed-V phase ends and arrives during that phase's fold.
 #pragma unroll
@@ -1122,7 +1258,9 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             for (int r0 = 0; r0 < R; r0 += kResTile) {
                 const bool more = r0 + kResTile < R;
                 const int r = r0 + krow;
-                load_res_v(r0, rv);   // the tile's value words: in flight while its logits and weights are worked out
+                // the tile's value words: in flight while its logits and weights are worked out (the first
+                // tile's may have been requested long before)
+                if (kResAhead2 < 2 || r0 > 0) load_res_v(r0, rv);
                 float dot[HPB];
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) {
