@@ -57,24 +57,7 @@ constexpr int kRegPair = 8;        // rounds of logits a thread of a 512-thread 
 constexpr int kRegTwoBit = 4;      // ... of the 2-bit kernel with four heads per unit (4 096 tokens)
 constexpr int kRegLong = 10;       // ... of a 1024-thread workgroup that holds a long chunk in one launch (10 240 tokens)
 constexpr float kLog2e = 1.4426950408889634f;
-#ifndef CQ_X_ROT
-#define CQ_X_ROT 1
-#endif
-#ifndef CQ_X_VPF
-#define CQ_X_VPF 1
-#endif
-#ifndef CQ_X_RES
-#define CQ_X_RES 0
-#endif
-#ifndef CQ_X_VREQ
-#define CQ_X_VREQ -1
-#endif
-#ifndef CQ_X_PRIO
-#define CQ_X_PRIO 1
-#endif
-#ifndef CQ_X_KENTRY
-#define CQ_X_KENTRY 0
-#endif
+
 
 template <int N> struct alignas(N * 4) Vec { float v[N]; };
 // native 16-byte vector: copies are single vector moves (HIP's uint4 struct copies lower to memcpy)
@@ -210,10 +193,10 @@ __device__ __forceinline__ void max_step(int* k) {
 }
 
 // Block-wide maximum of N values (integer keys, see float_key); result wave-uniform.
-// One barrier; `red` (kNW * N words) must not be rewritten before the next barrier of the caller.
+// One barrier; `red`: N words that hold the smallest key when the first wave gets here.
 template <int N, int kNW>
 __device__ __forceinline__ void block_max(float* v, float* red) {
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
     int* redi = reinterpret_cast<int*>(red);
     int k[N];
 #pragma unroll
@@ -224,25 +207,15 @@ __device__ __forceinline__ void block_max(float* v, float* red) {
     max_step<N, 0x140>(k);
     max_step<N, 0x142, 0xa>(k);
     max_step<N, 0x143, 0xc>(k);
+    // second stage: the waves' maxima meet in N words of LDS (set to the smallest key before the last barrier
+    // ahead of this call) through one atomic per wave and value
     if (lane == 63) {   // the last lane holds the wave's maxima
 #pragma unroll
-        for (int h = 0; h < N; ++h) redi[w * N + h] = k[h];
+        for (int h = 0; h < N; ++h) __hip_atomic_fetch_max(redi + h, k[h], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
     __syncthreads();
-    static_assert(kNW <= 16, "second stage folds at most 16 wave partials");
-    int x[N];
 #pragma unroll
-    for (int h = 0; h < N; ++h) x[h] = static_cast<int>(0x80000000u);
-    if (lane < kNW) {
-#pragma unroll
-        for (int h = 0; h < N; ++h) x[h] = redi[lane * N + h];
-    }
-    max_step<N, 0xB1>(x);   // lanes 0..15 hold the partials
-    max_step<N, 0x4E>(x);
-    max_step<N, 0x141>(x);
-    max_step<N, 0x140>(x);
-#pragma unroll
-    for (int h = 0; h < N; ++h) v[h] = key_float(__builtin_amdgcn_readfirstlane(x[h]));
+    for (int h = 0; h < N; ++h) v[h] = key_float(__builtin_amdgcn_readfirstlane(redi[h]));
 }
 
 // Unit decomposition of a 1-D grid.  Consecutive work ids share packed codes
@@ -304,8 +277,12 @@ __device__ __forceinline__ uint32_t pack_f16(float a, float b) {
 // none of their code.  EXTRAS: an additive mask or a residual row count read from device memory may be present; a
 // call with neither runs an instantiation without their code (32.6-32.8 against 33.5-34.0 us at the benchmark shape:
 // the kernel sits at the register limit of its occupancy, and code that never runs still costs registers).
+// NH: query heads a unit serves, at most HPB.  Tables, slots and partials are laid out HPB heads wide either way
+// (16-byte entries at HPB = 4); with NH = 3 the fourth lane of every entry is dead and the arithmetic on it is
+// left out - six query heads per kv-head (InternLM2-20B) make two exact units of three instead of two units of
+// four that carry two padding heads between them.
 template <int BITS, int HPB, typename DT, bool MINMAX_ONLY, bool VTOK = false, int NT = 1024, int REGL = 0,
-          bool CHUNKED = MINMAX_ONLY, bool EXTRAS = !MINMAX_ONLY>
+          bool CHUNKED = MINMAX_ONLY, bool EXTRAS = !MINMAX_ONLY, int NH = HPB>
 // (four waves per SIMD - at most 128 VGPRs - for either workgroup size: two 512-thread workgroups per compute
 // unit are only resident together within that)
 __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
@@ -344,23 +321,10 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
         constexpr int PH = decltype(phase_c)::value;   // 0 set-up and tables, 1 K look-ups, 2 min/max .. exp, 3 packed V, 4 folds, window, merge
         if constexpr (NT == 512) {
             if (prio_on) {
-#if CQ_X_PRIO == 1
                 if constexpr (PH == 0 || PH == 2) __builtin_amdgcn_s_setprio(2);
                 else if constexpr (PH == 1) { if (second) __builtin_amdgcn_s_setprio(0); else __builtin_amdgcn_s_setprio(1); }
                 else if constexpr (PH == 3) { if (second) __builtin_amdgcn_s_setprio(2); else __builtin_amdgcn_s_setprio(1); }
                 else __builtin_amdgcn_s_setprio(0);
-#elif CQ_X_PRIO == 2   // latency phases above the loops, loops equal
-                if constexpr (PH == 0 || PH == 2) __builtin_amdgcn_s_setprio(2);
-                else if constexpr (PH == 1 || PH == 3) __builtin_amdgcn_s_setprio(1);
-                else __builtin_amdgcn_s_setprio(2);
-#elif CQ_X_PRIO == 3   // as 1, tail phases high
-                if constexpr (PH == 0 || PH == 2) __builtin_amdgcn_s_setprio(2);
-                else if constexpr (PH == 1) { if (second) __builtin_amdgcn_s_setprio(0); else __builtin_amdgcn_s_setprio(1); }
-                else if constexpr (PH == 3) { if (second) __builtin_amdgcn_s_setprio(2); else __builtin_amdgcn_s_setprio(1); }
-                else __builtin_amdgcn_s_setprio(3);
-#elif CQ_X_PRIO == 4   // first workgroup ahead everywhere
-                if (second) __builtin_amdgcn_s_setprio(0); else __builtin_amdgcn_s_setprio(1);
-#endif
             }
         }
     };
@@ -374,8 +338,9 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
     qn = g.d_hkv.quot(vb);
     const int hkv = static_cast<int>(vb - qn * g.d_hkv.div);
     const int b = static_cast<int>(qn);
-    const int hq0 = hkv * G + hg * HPB;
-    const int nh = min(HPB, G - hg * HPB);   // query heads of this unit; the rest of its HPB heads are padding
+    static_assert(NH >= 1 && NH <= HPB, "heads per unit");
+    const int hq0 = hkv * G + hg * NH;
+    const int nh = min(NH, G - hg * NH);   // query heads of this unit; the rest of its NH heads are padding
     const int64_t bh = static_cast<int64_t>(b) * g.Hkv + hkv;
 
     const bool img_unit = split < g.nsplit && g.T > 0;
@@ -425,15 +390,6 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
     const U4* cvp4 = reinterpret_cast<const U4*>(cvp);
     const int last_u = has_img ? n * NB / 16 - 1 : 0;   // last valid 16-byte unit of either stream
     const int last_uk = k_rows ? last_u : 0;
-    uint4 kc[L::KR][BITS];
-    constexpr bool kKEntry = CQ_X_KENTRY && L::INA;
-    if constexpr (kKEntry) {
-#pragma unroll
-        for (int r = 0; r < L::KR; ++r) {
-#pragma unroll
-            for (int i = 0; i < BITS; ++i) kc[r][i] = ckp[min((tid + r * kNT) * BITS + i, last_uk)];
-        }
-    }
     // residual tile: K slice (row = tid / LPR, 128 / LPR elements); V: a wave owns RPW rows of the tile and a
     // lane one channel pair of each of them, so the value products need no fold inside the wave
     constexpr int LPR = L::LPR, NKP = L::NKP, RPW = L::RPW;
@@ -493,15 +449,17 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
         fx[L::F_VSZ + d] = Cvt<DT>::to_float(s_raw);
         fx[L::F_VSZ + kD + d] = Cvt<DT>::to_float(z_raw);
     }
+    if (tid < 3 * HPB) reinterpret_cast<int*>(red)[tid] = static_cast<int>(0x80000000u);   // block_max's meeting words
     // The packed K rows are requested only now: a wave that has to queue 64 KB of requests
     // first gets to phase 0 thousands of cycles later, and the table build below covers
     // their latency anyway.
-    if constexpr (!kKEntry) {
+    // (requested any later - after the table build, or all but the first round - the launch is slower;
+    // requested at kernel entry, ahead of q, as well)
+    uint4 kc[L::KR][BITS];
 #pragma unroll
-        for (int r = 0; r < L::KR; ++r) {
+    for (int r = 0; r < L::KR; ++r) {
 #pragma unroll
-            for (int i = 0; i < BITS; ++i) kc[r][i] = ckp[min((tid + r * kNT) * BITS + i, last_uk)];
-        }
+        for (int i = 0; i < BITS; ++i) kc[r][i] = ckp[min((tid + r * kNT) * BITS + i, last_uk)];
     }
     // Chunked launch: the chunks' logit min / max, lane s the pair of chunk s for every head (all in flight
     // together; they are folded across the wave where the calibration needs them), and - with a logits
@@ -532,7 +490,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
     float o_res = 0.f;
     float mn[HPB], mx[HPB];
 #pragma unroll
-    for (int h = 0; h < HPB; ++h) { mn[h] = INFINITY; mx[h] = -INFINITY; }
+    for (int h = 0; h < HPB; ++h) { mn[h] = h < NH ? INFINITY : 0.f; mx[h] = h < NH ? -INFINITY : 0.f; }
     // logits (later: calibrated, masked logits) of a token: in its slot, or in the thread's registers
     auto load_logits = [&](int rd, int tt) {
         if constexpr (REGL > 0) return lg[rd];
@@ -559,7 +517,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
     // rest as the K registers free up, so it has arrived when the logits are done.
     U4 vc[kPF];
     auto request_v = [&](int r) { vc[r] = cvp4[min((tid + (r / BITS) * kNT) * BITS + r % BITS, last_u)]; };
-    constexpr int kVEarly = (CQ_X_VREQ >= 0 && L::INA && L::KPASS == 1) ? 0 : kPF / 2;
+    constexpr int kVEarly = kPF / 2;
     if constexpr (!MINMAX_ONLY) {
 #pragma unroll
         for (int r = 0; r < kVEarly; ++r) request_v(r);
@@ -624,9 +582,27 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
         for (int i = 0; i < NBP / 4; ++i)
             pofs4[i] = pofs[4 * i] | (pofs[4 * i + 1] << 8) | (pofs[4 * i + 2] << 16) | (pofs[4 * i + 3] << 24);
         // c: the L::PCS 16-byte pieces of the row that pass P looks at; rd: the token's round (REGL)
+        // kLateMM (one table pass, logits in registers): a wave works out a round's logits for all its lanes as soon
+        // as its first lane has a token - the lanes past the chunk's end hold a copy of its last row (clamped
+        // request) and get that token's logits - so the min / max can be taken afterwards over the registers, two
+        // rounds per instruction, with no lane left out.
+        constexpr bool kLateMM = L::KPASS == 1 && REGL > 0 && !MINMAX_ONLY;
+        // a table entry: the NH live floats of it (12 bytes at three heads)
+        auto lds_entry = [&](uint32_t addr) {
+            V r;
+            if constexpr (NH == HPB) {
+                r = lds_floats<HPB>(addr);
+            } else {
+                typedef float VT __attribute__((ext_vector_type(NH)));
+                const VT v = *(const __attribute__((address_space(3))) VT*)(static_cast<uintptr_t>(addr));
+#pragma unroll
+                for (int k = 0; k < HPB; ++k) r.v[k] = k < NH ? v[k < NH ? k : 0] : 0.f;
+            }
+            return r;
+        };
         auto token_logits = [&](auto pass_c, int rd, int tt, const uint4* c) {
             constexpr int P = decltype(pass_c)::value;
-            if (tt < n) {
+            if (kLateMM ? (__builtin_amdgcn_readfirstlane(tt) < n) : (tt < n)) {
                 constexpr int WO = (P * L::WPP) % 4;   // the pass's first word inside its first piece
                 uint32_t w[NW32];
 #pragma unroll
@@ -657,7 +633,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                         // The kernel's only LDS object is the dynamic array, so it starts at LDS
                         // address 0 and the K table with it (the host checks that the kernel has no
                         // static LDS before the first launch): the permute result is the address.
-                        cur = lds_floats<HPB>(__builtin_amdgcn_perm(wds[k >> 2], pofs4[k >> 2], sel));
+                        cur = lds_entry(__builtin_amdgcn_perm(wds[k >> 2], pofs4[k >> 2], sel));
                     } else {
                         const uint32_t byte = (wds[k >> 2] >> (8 * (k & 3))) & 0xffu;
                         cur = *reinterpret_cast<const V*>(ktab_b + byte * (NBP * L::ESZ) + pofs[k]);
@@ -666,7 +642,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                     for (int l = 0; l < 6; ++l) {
                         if ((k >> l) & 1) {
 #pragma unroll
-                            for (int h = 0; h < HPB; ++h) cur.v[h] += part[l].v[h];
+                            for (int h = 0; h < NH; ++h) cur.v[h] += part[l].v[h];
                         } else {
                             part[l] = cur;
                             break;
@@ -680,15 +656,17 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                 if constexpr (P > 0) {   // add the earlier pass's partial
                     const V prev = load_logits(rd, tt);
 #pragma unroll
-                    for (int h = 0; h < HPB; ++h) acc.v[h] += prev.v[h];
+                    for (int h = 0; h < NH; ++h) acc.v[h] += prev.v[h];
                 }
+#pragma unroll
+                for (int h = NH; h < HPB; ++h) acc.v[h] = 0.f;   // dead lanes of the entry
                 if constexpr (!MINMAX_ONLY || P + 1 < L::KPASS) store_logits(rd, tt, acc);
                 if constexpr (MINMAX_ONLY && P + 1 == L::KPASS) {
                     if (g.lgt) gl[tt] = acc;   // for the main launch
                 }
-                if constexpr (P + 1 == L::KPASS) {
+                if constexpr (P + 1 == L::KPASS && !kLateMM) {
 #pragma unroll
-                    for (int h = 0; h < HPB; ++h) { mn[h] = fminf(mn[h], acc.v[h]); mx[h] = fmaxf(mx[h], acc.v[h]); }
+                    for (int h = 0; h < NH; ++h) { mn[h] = fminf(mn[h], acc.v[h]); mx[h] = fmaxf(mx[h], acc.v[h]); }
                 }
             }
         };
@@ -754,7 +732,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             // One table pass, logits in registers: the rows stream through the KR row registers - when a
             // round's row has been looked up its registers take the row of KR rounds later, so KR rounds
             // are in flight while one is worked on and no batch of rows is waited for as a whole.
-            constexpr bool kRotate = CQ_X_ROT && L::KPASS == 1 && REGL > 0;
+            constexpr bool kRotate = L::KPASS == 1 && REGL > 0;
             if constexpr (kRotate) {
                 static_assert(!kRotate || BITS == 1, "one 16-byte piece per row");
 #pragma unroll
@@ -762,8 +740,23 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                     token_logits(pass_c, rd, tid + rd * kNT, kc[rd % L::KR]);
                     if (rd + L::KR < REGL) kc[rd % L::KR][0] = ckp[min(tid + (rd + L::KR) * kNT, last_uk)];
                     if constexpr (!MINMAX_ONLY) {
-                        if constexpr (CQ_X_VREQ >= 0) { if (rd >= CQ_X_VREQ && rd < CQ_X_VREQ + kPF) request_v(rd - CQ_X_VREQ); }
-                        else if (rd < kPF - kVEarly) request_v(kVEarly + rd);   // the rest of the first packed V block
+                        if (rd < kPF - kVEarly) request_v(kVEarly + rd);   // the rest of the first packed V block
+                    }
+                }
+                if constexpr (kLateMM) {
+                    const int t0w = __builtin_amdgcn_readfirstlane(tid);   // the wave's first token of round 0
+#pragma unroll
+                    for (int rd = 0; rd < REGL; rd += 2) {
+                        if (rd + 1 < REGL && t0w + (rd + 1) * kNT < n) {
+#pragma unroll
+                            for (int h = 0; h < NH; ++h) {
+                                mn[h] = fminf(mn[h], fminf(lg[rd].v[h], lg[rd + 1].v[h]));
+                                mx[h] = fmaxf(mx[h], fmaxf(lg[rd].v[h], lg[rd + 1].v[h]));
+                            }
+                        } else if (t0w + rd * kNT < n) {
+#pragma unroll
+                            for (int h = 0; h < NH; ++h) { mn[h] = fminf(mn[h], lg[rd].v[h]); mx[h] = fmaxf(mx[h], lg[rd].v[h]); }
+                        }
                     }
                 }
                 return;
@@ -912,13 +905,10 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                     stage_piece(vc[r], tok, r % BITS, tok < vn0);
                 }
             }
-            // The registers of the staged block take the next block's rows right away (clamped addresses when
-            // there is none), and the first residual tile is requested behind them: everything the rest of the
-            // unit reads is in flight while the exponentials and the packed-V loop run, instead of each stream
-            // being asked for when its phase starts - all workgroups of a launch reach their phases together, and
-            // the memory system would idle through the vector-bound phases and then see every request at once.
-            constexpr bool kVAhead = CQ_X_VPF && L::INA;
-            constexpr int kResAhead = L::INA ? CQ_X_RES : 0;
+            // The registers of a staged block take the next block's rows (clamped addresses when there is none):
+            // the block is in flight while the current one is multiplied, instead of being asked for behind a
+            // barrier when the loop gets there.  (The first residual tile requested here as well measured slower.)
+            constexpr bool kVAhead = L::INA;
             auto request_v_block = [&](int vs0) {
 #pragma unroll
                 for (int r = 0; r < kPF; ++r) vc[r] = cvp4[min((vs0 + tid + (r / BITS) * kNT) * BITS + r % BITS, last_u)];
@@ -949,7 +939,8 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                 if (g.calib) {
                     const float tgt_max = mx[h] + g.off_max;
                     tmin[h] = mn[h] + g.off_min;
-                    slope[h] = (tgt_max - tmin[h]) / (mx[h] - mn[h] + 1e-8f);
+                    // (the hardware reciprocal, one unit in the last place: far inside the tolerance of the map)
+                    slope[h] = (tgt_max - tmin[h]) * __builtin_amdgcn_rcpf(mx[h] - mn[h] + 1e-8f);
                 } else {
                     tmin[h] = mn[h];
                     slope[h] = 1.0f;
@@ -970,7 +961,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                     }
                     store_logits(rd, tt, w);
                 });
-                block_max<HPB, kNW>(lm, red + kNW * 2 * HPB);   // the first reduction's words may still be read
+                block_max<HPB, kNW>(lm, red + 2 * HPB);   // words of its own
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) { m_img[h] = lm[h]; slope[h] = 1.0f; tmin[h] = 0.f; mn[h] = 0.f; }
             } else {
@@ -995,16 +986,27 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             float cma[VTOK ? L::NGRP * HPB : 1];   // sum_t e[t][h] * minimum[t][group], kept [group][head]
 #pragma unroll
             for (int i = 0; i < (VTOK ? L::NGRP * HPB : 1); ++i) cma[i] = 0.f;
+            // With a slope of ordinary size the subtraction folds into the constant: exp2(w * ea + (ec - mn * ea)), one
+            // FMA per logit.  A degenerate logit range makes the slope ~1e8, and only the exact zero of (w - mn)
+            // keeps the product finite: those units take the two-step form.
+            float ec2[HPB];
+            bool plain = true;
+#pragma unroll
+            for (int h = 0; h < HPB; ++h) {
+                ec2[h] = ec[h] - mn[h] * ea[h];
+                if (h < NH) plain = plain && fabsf(ea[h]) <= 4.0f;
+            }
+            auto exp_tokens = [&](auto fused_c) {
+            constexpr bool kFused = decltype(fused_c)::value;
             for_my_tokens(npad, [&](int rd, int tt) {
                 float e[4] = {0.f, 0.f, 0.f, 0.f};
                 uint32_t sc2[2] = {0u, 0u};   // the token's group scales as fp16
                 if (tt < n) {
                     const V w = load_logits(rd, tt);
 #pragma unroll
-                    for (int h = 0; h < HPB; ++h) {
-                        // (w - mn) first: with a degenerate logit range the slope is ~1e8 and only the exact
-                        // zero of the difference keeps the product finite
-                        e[h] = __builtin_amdgcn_exp2f((w.v[h] - mn[h]) * ea[h] + ec[h]);
+                    for (int h = 0; h < NH; ++h) {
+                        if constexpr (kFused) e[h] = __builtin_amdgcn_exp2f(__builtin_fmaf(w.v[h], ea[h], ec2[h]));
+                        else e[h] = __builtin_amdgcn_exp2f((w.v[h] - mn[h]) * ea[h] + ec[h]);
                         ls[h] += e[h];
                     }
                     if constexpr (VTOK) {
@@ -1026,14 +1028,15 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                 *reinterpret_cast<HWv*>(slot(tt)) = hw;
                 if constexpr (VTOK) *reinterpret_cast<uint2*>(slot(tt) + 8) = make_uint2(sc2[0], sc2[1]);
             });
+            };
+            if (plain) exp_tokens(std::true_type{});
+            else exp_tokens(std::false_type{});
             // The sums of e (and of e * minimum) are only needed at the very end: each thread
             // keeps its partial through the packed-V phase and the fold rides on that phase's
             // closing barriers.
             __syncthreads();   // publishes e and vst
             // (requested here, not right after the staging: the logits' registers are free now)
             if constexpr (kVAhead) request_v_block(L::VSUB);
-            if constexpr (kResAhead >= 1) load_res_k(0, rk);
-            if constexpr (kResAhead >= 2) load_res_v(0, rv);
 
             // ---- phase 5: packed V ----------------------------------------------------------
             // lane = (byte column j, slice c of its 8 bit lanes); a wave pass covers TPW tokens
@@ -1089,7 +1092,9 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                     if constexpr (kVAhead) request_v_block(vs0 + L::VSUB);
                     __syncthreads();
                 }
-                for (int u = wvu; u * L::TPW < vn; u += kNW) {   // wave-uniform loop control
+                // One pass over the TPW tokens of unit u: the sum of the entries each of the lane's bit lanes picks,
+                // as packed fp16 (GPW entries of at most 4 terms each, added pairwise).
+                auto v_pass = [&](int u, f16x2_t (&sum)[L::MPL][L::HW]) {
                     const int tl = u * L::TPW;        // token offset inside the block
                     if (bg < L::GPW) {
                         // entry `be` of group `bg`: fp16 sum of the e values its bits select
@@ -1156,18 +1161,44 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
 #pragma unroll
                                 for (int k = 0; k < L::HW; ++k) pk[m][gq][k] += pk[m][gq + st][k];
 #pragma unroll
-                        for (int h = 0; h < HPB; ++h) {
-                            const f16x2_t pr = pk[m][0][h >> 1];
-                            const _Float16 hv = (h & 1) ? pr.y : pr.x;
-                            acc[m][h] = __builtin_fmaf(static_cast<float>(hv), one, acc[m][h]);
-                        }
+                        for (int k = 0; k < L::HW; ++k) sum[m][k] = pk[m][0][k];
                     }
                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                     __builtin_amdgcn_wave_barrier();
+                };
+                // one mixed-precision FMA per head moves a packed sum into the fp32 accumulators
+                auto v_flush = [&](const f16x2_t (&sum)[L::MPL][L::HW]) {
+#pragma unroll
+                    for (int m = 0; m < L::MPL; ++m)
+#pragma unroll
+                        for (int h = 0; h < NH; ++h) {
+                            const f16x2_t pr = sum[m][h >> 1];
+                            const _Float16 hv = (h & 1) ? pr.y : pr.x;
+                            acc[m][h] = __builtin_fmaf(static_cast<float>(hv), one, acc[m][h]);
+                        }
+                };
+                int u = wvu;   // wave-uniform loop control
+                {
+                    // two passes per fp32 accumulation: the sums of 2 * TPW tokens meet as packed fp16 first
+                    for (; (u + kNW) * L::TPW < vn; u += 2 * kNW) {
+                        f16x2_t s0[L::MPL][L::HW], s1[L::MPL][L::HW];
+                        v_pass(u, s0);
+                        v_pass(u + kNW, s1);
+#pragma unroll
+                        for (int m = 0; m < L::MPL; ++m)
+#pragma unroll
+                            for (int k = 0; k < L::HW; ++k) s0[m][k] += s1[m][k];
+                        v_flush(s0);
+                    }
+                }
+                for (; u * L::TPW < vn; u += kNW) {
+                    f16x2_t s0[L::MPL][L::HW];
+                    v_pass(u, s0);
+                    v_flush(s0);
                 }
             }
             phase_priority(std::integral_constant<int, 4>{});
-            if constexpr (kResAhead < 1) load_res_k(0, rk);   // first residual tile's K rows: in flight during the fold below
+            load_res_k(0, rk);   // first residual tile's K rows: in flight during the fold below
             // per-wave partial sums of e (and of e * minimum), folded by the output threads below
             constexpr int kSums = VTOK ? (L::NGRP + 1) * HPB : HPB;
             wave_reduce_n<HPB>(ls, OpSum(), 0.f);
@@ -1228,11 +1259,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             __syncthreads();
         }
 
-        constexpr int kResAhead2 = L::INA ? CQ_X_RES : 0;
-        if (n == 0) {
-            load_res_k(0, rk);
-            if constexpr (kResAhead2 >= 2) load_res_v(0, rv);
-        }
+        if (n == 0) load_res_k(0, rk);
         // ---- phase 6: full-precision residual rows, online softmax.  Runs last: its first
         // tile is requested when the packed-V phase ends and arrives during that phase's fold.
 #pragma unroll
@@ -1258,12 +1285,12 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             for (int r0 = 0; r0 < R; r0 += kResTile) {
                 const bool more = r0 + kResTile < R;
                 const int r = r0 + krow;
-                // the tile's value words: in flight while its logits and weights are worked out (the first
-                // tile's may have been requested long before)
-                if (kResAhead2 < 2 || r0 > 0) load_res_v(r0, rv);
+                load_res_v(r0, rv);   // the tile's value words: in flight while its logits and weights are worked out
                 float dot[HPB];
 #pragma unroll
-                for (int h = 0; h < HPB; ++h) {
+                for (int h = NH; h < HPB; ++h) dot[h] = 0.f;
+#pragma unroll
+                for (int h = 0; h < NH; ++h) {
                     float a = 0.f;
 #pragma unroll
                     for (int i = 0; i < NKP; ++i) {
@@ -1283,7 +1310,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                     for (int h = 0; h < HPB; ++h) sres[krow * HPB + h] = (r < R) ? dot[h] + mv : -INFINITY;
                 }
                 __syncthreads();
-                if (wv < HPB) {   // wave h keeps the running softmax state of head h
+                if (wv < NH) {   // wave h keeps the running softmax state of head h
                     const int h = wv;
                     constexpr int kRL = kResTile / kWave;   // tile rows per lane
                     float sv[kRL], smax = -INFINITY;
@@ -1309,7 +1336,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                 __syncthreads();
                 if (r0 > 0) {
 #pragma unroll
-                    for (int h = 0; h < HPB; ++h) {
+                    for (int h = 0; h < NH; ++h) {
                         const float al = stat[h];
                         accv[0][h] *= al;
                         accv[1][h] *= al;
@@ -1320,7 +1347,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                     const float f0 = Cvt<DT>::lo(rv[i]), f1 = Cvt<DT>::hi(rv[i]);
                     const V p = reinterpret_cast<const V*>(pres)[wvr * RPW + i];   // the row's weights (0 past R), one address per wave
 #pragma unroll
-                    for (int h = 0; h < HPB; ++h) {
+                    for (int h = 0; h < NH; ++h) {
                         accv[0][h] = __builtin_fmaf(p.v[h], f0, accv[0][h]);
                         accv[1][h] = __builtin_fmaf(p.v[h], f1, accv[1][h]);
                     }
@@ -1362,7 +1389,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                 const float wr = (mr == -INFINITY) ? 0.f : __expf(mr - mf);
                 const float num = o_img * wi + o_res * wr;
                 const float den = li * wi + lr * wr;
-                store_elem<DT>(g.out, row * kD + d, num / den);
+                store_elem<DT>(g.out, row * kD + d, num * __builtin_amdgcn_rcpf(den));
             } else {
                 float* p = g.part + (row * g.nx + split) * (kD + 2);
                 const bool is_img = split < g.nsplit;
@@ -1440,15 +1467,15 @@ static int pair_units() {
 static inline int ngroups(int G, int hpb) { return (G + hpb - 1) / hpb; }
 
 struct Plan {
-    int hpb, nt, regl, nsplit, chunk, nx, cap, lds;
+    int hpb, nh, nt, regl, nsplit, chunk, nx, cap, lds;   // hpb: heads an entry is wide; nh: heads a unit serves
     size_t ws_mm, ws_part, ws_cnt, ws_lgt;   // chunked launch: min / max, partials, counters; logits (optional)
 };
 
 template <int BITS, int HPB, bool VTOK, int NT = 1024, int REGL = 0>
-static void plan_for(const cq_decode_args* a, Plan* p) {
+static void plan_for(const cq_decode_args* a, Plan* p, int nh = HPB) {
     using L = Lay<BITS, HPB, VTOK, NT, REGL>;
     const int G = a->Hq / a->Hkv;
-    const int64_t units = static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, HPB);
+    const int64_t units = static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, nh);
     const int maxc = L::max_chunk();
     int nsplit = 1;
     if (a->T > 0) {
@@ -1470,6 +1497,7 @@ static void plan_for(const cq_decode_args* a, Plan* p) {
     if (chunk > maxc) chunk = maxc;
     nsplit = a->T > 0 ? (a->T + chunk - 1) / chunk : 1;
     p->hpb = HPB;
+    p->nh = nh;
     p->nt = NT;
     p->regl = REGL;
     p->nsplit = nsplit;
@@ -1500,11 +1528,14 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
     const int G = a->Hq / a->Hkv;
     if (a->v_mode != CQ_V_PER_CHANNEL && a->v_mode != CQ_V_PER_TOKEN) return CQ_ERR_UNSUPPORTED;
     const bool vtok = a->v_mode == CQ_V_PER_TOKEN;
+    // heads a unit with four-wide entries serves: three when that divides the group exactly and four does not
+    // (G = 3, 6, 9: exact units instead of a padded last one; per-channel values only)
+    const int nh4 = (!vtok && G % 3 == 0 && G % 4 != 0) ? 3 : 4;
     if (a->bits == 1) {
         // G = 3, 5, 6, 7, ...: units of four heads with the last one partly padding (two units per kv head at
         // G = 6) do less work than units of two heads or one (three or six of them, each walking all the packed rows)
         const bool pad4 = G % 4 != 0 && G > 2;
-        if (G % 4 == 0 || pad4) vtok ? plan_for<1, 4, true>(a, p) : plan_for<1, 4, false>(a, p);
+        if (G % 4 == 0 || pad4) vtok ? plan_for<1, 4, true>(a, p) : plan_for<1, 4, false>(a, p, nh4);
         else if (G % 2 == 0) vtok ? plan_for<1, 2, true>(a, p) : plan_for<1, 2, false>(a, p);
         else vtok ? plan_for<1, 1, true>(a, p) : plan_for<1, 1, false>(a, p);
         // More units than compute units: 512-thread workgroups, two resident per compute unit, need fewer
@@ -1514,17 +1545,17 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
         // the token slots: with the logits in registers (half the bytes per token slot) the layout may still
         // hold all T tokens in one launch, which saves the min/max launch's second pass over the packed K rows.
         if (p->hpb == 4 && !vtok && a->force_splits == 0 && p->nsplit > 1 &&
-            static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, 4) >= kPairUnits * 3 / 4) {
+            static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, nh4) >= kPairUnits * 3 / 4) {
             Plan q;
-            plan_for<1, 4, false, 1024, kRegLong>(a, &q);
+            plan_for<1, 4, false, 1024, kRegLong>(a, &q, nh4);
             if (q.nsplit == 1) *p = q;
         }
         // Single launch: only if the 512-thread layout also holds all T tokens.  Chunked launch (four heads
         // per unit): the chunks are units of their own.
-        const int64_t units = static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, p->hpb);
+        const int64_t units = static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, p->nh);
         if (!vtok && a->force_splits == 0 && p->hpb >= 2) {
             Plan q;
-            if (p->hpb == 4) plan_for<1, 4, false, 512, kRegPair>(a, &q); else plan_for<1, 2, false, 512, 0>(a, &q);
+            if (p->hpb == 4) plan_for<1, 4, false, 512, kRegPair>(a, &q, nh4); else plan_for<1, 2, false, 512, 0>(a, &q);
             const bool single = p->nsplit == 1 && q.nsplit == 1 && units > kPairUnits;
             const bool chunked = p->hpb == 4 && p->nsplit > 1 && q.nsplit > 1 && units * q.nsplit > kPairUnits;
             if ((single || chunked) && q.lds <= kLdsMax / 2) *p = q;
@@ -1534,12 +1565,12 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
         // would not hold a 3 328-token chunk, so that mode keeps two heads per unit
         // (the first pass's partial logits wait in registers, four tokens per thread: -3 % against the token slots)
         if ((G % 4 == 0 || G > 2) && !vtok) {
-            plan_for<2, 4, false, 1024, kRegTwoBit>(a, p);
-            // more units than compute units: two 512-thread workgroups per compute unit (K table in four passes)
-            const int64_t units = static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, 4);
+            plan_for<2, 4, false, 1024, kRegTwoBit>(a, p, nh4);
+            // more units than compute units: two 512-thread workgroups per compute unit (K table in two passes)
+            const int64_t units = static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, nh4);
             if (a->force_splits == 0) {
                 Plan q;
-                plan_for<2, 4, false, 512, kRegPair>(a, &q);
+                plan_for<2, 4, false, 512, kRegPair>(a, &q, nh4);
                 const bool single = p->nsplit == 1 && q.nsplit == 1 && units > kPairUnits;
                 const bool chunked = p->nsplit > 1 && q.nsplit > 1 && units * q.nsplit > kPairUnits;
                 if ((single || chunked) && q.lds <= kLdsMax / 2) *p = q;
@@ -1552,7 +1583,7 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
     // heads per unit make the units cheaper (18.8 / 15.5 / 14.2 us for four / two / one head at 3 328 + 128 tokens)
     // and there are compute units for two or four times as many of them.
     if (a->force_splits == 0 && p->nsplit == 1 && p->hpb == 4) {
-        const int64_t u4 = static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, 4);
+        const int64_t u4 = static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, p->nh);
         const int h = u4 <= 32 ? 1 : (u4 <= 64 && G % 2 == 0) ? 2 : 4;
         Plan q = *p;
         if (a->bits == 1) {
@@ -1564,21 +1595,21 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
         }
         if (q.nsplit == 1) *p = q;
     }
-    const int64_t blocks = static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, p->hpb) * p->nx;
+    const int64_t blocks = static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, p->nh) * p->nx;
     if (blocks > 0x7fffffff) return CQ_ERR_SHAPE;
     return CQ_OK;
 }
 
-template <int BITS, int HPB, typename DT, bool VTOK, int NT = 1024, int REGL = 0>
+template <int BITS, int HPB, typename DT, bool VTOK, int NT = 1024, int REGL = 0, int NH = HPB>
 static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
     const int G = g.Hq / g.Hkv;
-    const unsigned units = static_cast<unsigned>(g.B) * g.Hkv * ngroups(G, HPB);
+    const unsigned units = static_cast<unsigned>(g.B) * g.Hkv * ngroups(G, NH);
     const bool extras = g.mask != nullptr || g.r_dev != nullptr;
-    auto kmain = g.nsplit > 1 ? (extras ? decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, true, true>
-                                        : decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, true, false>)
-                              : (extras ? decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, false, true>
-                                        : decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, false, false>);
-    auto kmm = decode_kernel<BITS, HPB, DT, true, false, NT, REGL>;   // the min/max pass never looks at values
+    auto kmain = g.nsplit > 1 ? (extras ? decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, true, true, NH>
+                                        : decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, true, false, NH>)
+                              : (extras ? decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, false, true, NH>
+                                        : decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, false, false, NH>);
+    auto kmm = decode_kernel<BITS, HPB, DT, true, false, NT, REGL, true, false, NH>;   // the min/max pass never looks at values
     // raise the dynamic-LDS limit once per device for this instantiation
     static std::atomic<uint32_t> attr_done{0};
     int dev = 0;
@@ -1586,10 +1617,10 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
     const uint32_t bit = 1u << (dev & 31);
     if (!(attr_done.load(std::memory_order_acquire) & bit)) {
         // the K look-ups address the table absolutely: the dynamic LDS array must start at 0
-        const void* kernels[5] = {reinterpret_cast<const void*>(decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, false, false>),
-                                  reinterpret_cast<const void*>(decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, false, true>),
-                                  reinterpret_cast<const void*>(decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, true, false>),
-                                  reinterpret_cast<const void*>(decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, true, true>),
+        const void* kernels[5] = {reinterpret_cast<const void*>(decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, false, false, NH>),
+                                  reinterpret_cast<const void*>(decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, false, true, NH>),
+                                  reinterpret_cast<const void*>(decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, true, false, NH>),
+                                  reinterpret_cast<const void*>(decode_kernel<BITS, HPB, DT, false, VTOK, NT, REGL, true, true, NH>),
                                   reinterpret_cast<const void*>(kmm)};
         for (const void* k : kernels) {
             hipFuncAttributes fa;
@@ -1604,7 +1635,7 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
     // (a main launch that reads its logits back has no look-up phase for the first workgroup to get ahead in:
     // with the priorities the second one would hold the packed-V loop to itself)
     gm.ncu = (NT == 512 && !g.lgt && static_cast<int64_t>(units) * g.nx <= 2 * static_cast<int64_t>(pair_units())) ? pair_units() : 0;
-    gm.d_ng.set(static_cast<uint32_t>(ngroups(G, HPB)));
+    gm.d_ng.set(static_cast<uint32_t>(ngroups(G, NH)));
     gm.d_nx.set(static_cast<uint32_t>(g.nx));
     gm.d_hkv.set(static_cast<uint32_t>(g.Hkv));
     if (g.nsplit > 1) {
@@ -1624,6 +1655,17 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
 
 template <typename DT, bool VTOK>
 static int dispatch(const DecodeGeom& g, const Plan& p, int bits, hipStream_t st) {
+    if constexpr (!VTOK) {
+        if (p.nh == 3 && p.hpb == 4) {   // exact units of three heads
+            if (bits == 1) {
+                if (p.nt == 512) return launch<1, 4, DT, false, 512, kRegPair, 3>(g, p, st);
+                if (p.regl) return launch<1, 4, DT, false, 1024, kRegLong, 3>(g, p, st);
+                return launch<1, 4, DT, false, 1024, 0, 3>(g, p, st);
+            }
+            if (p.nt == 512) return launch<2, 4, DT, false, 512, kRegPair, 3>(g, p, st);
+            return launch<2, 4, DT, false, 1024, kRegTwoBit, 3>(g, p, st);
+        }
+    }
     if (bits == 1) {
         if constexpr (!VTOK) {
             if (p.hpb == 4 && p.nt == 512) return launch<1, 4, DT, false, 512, kRegPair>(g, p, st);
@@ -1740,7 +1782,7 @@ int cq_decode_attn_plan(const cq_decode_args* args, cq_decode_plan* plan) {
     const int rc = cq::make_plan(args, &p);
     if (rc != CQ_OK) return rc;
     plan->threads = p.nt;
-    plan->heads_per_unit = p.hpb;
+    plan->heads_per_unit = p.nh;
     plan->chunks = p.nsplit;
     plan->chunk_tokens = args->T > 0 ? p.chunk : 0;
     plan->launches = p.nsplit > 1 ? 2 : 1;

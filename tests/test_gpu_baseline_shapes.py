@@ -63,10 +63,10 @@ def test_layer_shape_one_bit_batch_64_with_system_rows(ops):
 
 
 def test_26b_layer_shape_batch_16(ops):
-    """48 query / 8 kv heads, 9 984 packed tokens + 64 window rows: padded four-head units that hold the
-    whole token axis in one launch with the logits in registers."""
+    """48 query / 8 kv heads, 9 984 packed tokens + 64 window rows: two exact units of three heads per kv
+    head that hold the whole token axis in one launch with the logits in registers."""
     _repeated(ops, 2, 8, 48, 8, 9984, 64, 0, 1, seed=303,
-              expect_plan={"launches": 1, "heads_per_unit": 4, "register_logits": 10})
+              expect_plan={"launches": 1, "heads_per_unit": 3, "register_logits": 10})
 
 
 def test_long_context_batch_8_kv_32768(ops):

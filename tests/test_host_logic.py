@@ -44,7 +44,7 @@ def test_decode_launch_plan_is_a_function_of_the_shape():
     assert bench["lds_bytes"] <= 80 * 1024 and bench["chunk_tokens"] == 3328
     small = plan(32, 32, 8, 3328, 128)                       # 256 units: one 1024-thread workgroup per compute unit
     assert (small["threads"], small["register_logits"], small["launches"]) == (1024, 0, 1)
-    two_bit = plan(64, 32, 8, 3328, 128, bits=2)            # 2 bits: paired as well, K table in four passes
+    two_bit = plan(64, 32, 8, 3328, 128, bits=2)            # 2 bits: paired as well, K table in two passes
     assert (two_bit["threads"], two_bit["register_logits"]) == (512, 8) and two_bit["lds_bytes"] <= 80 * 1024
     assert plan(32, 32, 8, 3328, 128, bits=2)["threads"] == 1024
     assert plan(64, 32, 8, 3328, 128, v_mode=1)["threads"] == 1024
@@ -54,8 +54,11 @@ def test_decode_launch_plan_is_a_function_of_the_shape():
     long = plan(8, 32, 8, 32768, 0)                          # chunked: the chunks are the units
     assert long["launches"] == 2 and long["threads"] == 512 and long["chunks"] * long["chunk_tokens"] >= 32768
     assert long["lds_bytes"] <= 80 * 1024
-    big = plan(16, 48, 8, 9984, 64)     # six heads per kv head: two units of four (the second half padding); one launch
-    assert (big["threads"], big["heads_per_unit"], big["launches"], big["register_logits"]) == (1024, 4, 1, 10)   # logits in registers
+    big = plan(16, 48, 8, 9984, 64)     # six heads per kv head: two exact units of three; one launch
+    assert (big["threads"], big["heads_per_unit"], big["launches"], big["register_logits"]) == (1024, 3, 1, 10)   # logits in registers
+    assert plan(64, 48, 8, 3328, 128)["heads_per_unit"] == 3 and plan(64, 48, 8, 3328, 128)["threads"] == 512
+    assert plan(64, 24, 8, 3328, 128, bits=2)["heads_per_unit"] == 3      # three heads per kv head: one exact unit
+    assert plan(64, 40, 8, 3328, 128)["heads_per_unit"] == 4              # five: units of 4 + 1
     assert big["lds_bytes"] <= 160 * 1024
     tok = plan(16, 48, 8, 9984, 64, v_mode=1)               # per-token values: padded four-head units too, chunked (16-byte slots)
     assert (tok["heads_per_unit"], tok["threads"], tok["register_logits"]) == (4, 1024, 0) and tok["launches"] == 2
@@ -85,7 +88,9 @@ def test_decode_launch_plan_invariants_over_random_shapes():
         p = _lib.DecodePlan()
         assert lib.cq_decode_attn_plan(ctypes.byref(a), ctypes.byref(p)) == 0
         shape = (a.B, a.Hq, a.Hkv, a.T, a.R, a.bits, a.v_mode, a.force_splits)
-        assert p.threads in (512, 1024) and p.heads_per_unit in (1, 2, 4), shape
+        assert p.threads in (512, 1024) and p.heads_per_unit in (1, 2, 3, 4), shape
+        G_ = a.Hq // a.Hkv
+        assert (p.heads_per_unit == 3) <= (G_ % 3 == 0 and G_ % 4 != 0 and a.v_mode == 0), shape   # three only for exact units
         assert 0 < p.lds_bytes <= (80 if p.threads == 512 else 160) * 1024, shape
         assert p.chunks >= 1 and p.chunks * p.chunk_tokens >= a.T, shape
         assert p.chunk_tokens % 64 == 0, shape
