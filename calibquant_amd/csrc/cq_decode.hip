@@ -80,6 +80,19 @@ struct DecodeGeom {
                   // launch instead of its own K look-ups; NULL: the main launch recomputes them
     int* cnt;     // chunked launch: [unit] count of the unit's chunks (+ residual unit) that have written their
                   // partial; the one that finds all the others done merges them
+    // Chunked step in ONE launch (every chunk's workgroup resident at once): the chunks of a unit exchange their
+    // logit min / max inside the launch.  rec: [unit][head][chunk][2] 64-bit records, a float (min, then max)
+    // in the lower half and the call's epoch in the upper half - a record is valid by itself, so a chunk
+    // publishes with plain write-through stores and waits for nothing, and the others poll the records
+    // (whatever an earlier call or an uninitialised workspace left there has another epoch).  done64: [unit]
+    // partials written, tagged with the epoch the same way.  status: host-visible word that a workgroup sets
+    // when it gives up waiting (spin_limit polls); NULL: nowhere to report.
+    unsigned long long* rec;
+    unsigned long long* done64;
+    int* status;
+    uint32_t epoch;
+    int fused;
+    int spin_limit;
     int B, Hq, Hkv, T, R, S;
     int nsplit, chunk, nx;
     int calib;
@@ -264,6 +277,31 @@ template <int N> __device__ __forceinline__ Vec<N> lds_floats(uint32_t addr) {
 // A float handed from one workgroup to another inside a launch: device-scope atomic store.
 __device__ __forceinline__ void publish(float* p, float v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// One more arrival at an epoch-tagged counter; returns the arrivals of this epoch including this one.
+// SCOPE: device scope (the exchange is done where all dies see it), or workgroup scope, which this hardware
+// executes in the L2 of the issuing die like every read-modify-write - the fast form, for counters that only
+// workgroups of one die touch.
+// The current value of a 64-bit word as the L2 (or, at device scope, the memory side) holds it: a compare-and-
+// swap of 0 for 0.  (Not a read-modify-write that changes nothing, such as OR 0: the compiler turns those into
+// plain loads, which a compute unit's own cache may answer with what it read earlier.)
+template <int SCOPE>
+__device__ __forceinline__ unsigned long long peek64(unsigned long long* c) {
+    unsigned long long v = 0ull;
+    __hip_atomic_compare_exchange_strong(c, &v, 0ull, __ATOMIC_RELAXED, __ATOMIC_RELAXED, SCOPE);
+    return v;
+}
+
+template <int SCOPE>
+__device__ __forceinline__ uint32_t arrive(unsigned long long* c, uint32_t epoch) {
+    unsigned long long old = peek64<SCOPE>(c);
+    for (;;) {   // every failed exchange is another workgroup's success: at most as many rounds as workgroups
+        const unsigned long long want = (static_cast<uint32_t>(old >> 32) == epoch)
+                                            ? old + 1 : ((static_cast<unsigned long long>(epoch) << 32) | 1u);
+        if (__hip_atomic_compare_exchange_strong(c, &old, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED, SCOPE))
+            return static_cast<uint32_t>(want);
+    }
 }
 
 __device__ __forceinline__ uint32_t pack_f16(float a, float b) {
@@ -469,7 +507,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
     // REGL: the logits of this thread's tokens, round r = token tid + r * kNT
     V lg[REGL > 0 ? REGL : 1];
     if constexpr (!MINMAX_ONLY) {
-        if (CHUNKED && has_img) {
+        if (CHUNKED && has_img && !g.fused) {
 #pragma unroll
             for (int h = 0; h < HPB; ++h) {
                 const MinMax* p = reinterpret_cast<const MinMax*>(g.mm) +
@@ -869,6 +907,20 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
         for (int h = 0; h < HPB; ++h) m_img[h] = -INFINITY;
         float o_img = 0.f;  // thread (h, d) = (tid / kD, tid % kD) for tid < HPB*kD
 
+        if constexpr (CHUNKED) {
+            // One launch: this chunk's min / max go out now (write-through stores, waited for, then the arrival
+            // count); the other chunks' are collected further down, after the staging of the first V block.
+            if (g.fused && k_rows && tid == 0) {
+                unsigned long long* o = g.rec + ((unit * HPB) * g.nsplit + split) * 2;
+                const unsigned long long tag = static_cast<unsigned long long>(g.epoch) << 32;
+#pragma unroll
+                for (int h = 0; h < HPB; ++h) {
+                    __hip_atomic_store(o + h * g.nsplit * 2, tag | __float_as_uint(mn[h]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(o + h * g.nsplit * 2 + 1, tag | __float_as_uint(mx[h]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+        }
+
         if (n > 0) {
             // The K table is dead: stage the first block of packed V rows in its place
             // (ordered by the barrier of block_max).  Layout: [unit of TPW tokens]
@@ -915,7 +967,45 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             };
 
             // ---- phase 4: calibration + exp ---------------------------------------------
-            if constexpr (CHUNKED) {   // one fold for both: max of (-min, max) over the chunks
+            if constexpr (CHUNKED) {
+                if (g.fused) {
+                    // Wait until every chunk of the unit has published: the first wave polls the records, lane s
+                    // those of chunk s, a bounded number of times (workgroups that are not all resident together -
+                    // a smaller device than planned for - must not spin for ever; giving up ends this workgroup
+                    // without a result and tells the host), folds them and leaves the unit's min / max in LDS.
+                    float* fold = red + 4 * HPB;           // 2 * HPB floats, then the verdict
+                    int* flag = reinterpret_cast<int*>(fold + 2 * HPB);
+                    if (wv == 0) {
+                        const unsigned long long* pr = g.rec + ((unit * HPB) * g.nsplit + min(lane, g.nsplit - 1)) * 2;
+                        float mm2[2 * HPB];
+                        bool ok = false;
+                        for (int it = 0; it < g.spin_limit && !ok; ++it) {
+                            bool valid = true;
+#pragma unroll
+                            for (int h = 0; h < HPB; ++h) {
+                                const unsigned long long lo = __hip_atomic_load(pr + h * g.nsplit * 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                const unsigned long long hi = __hip_atomic_load(pr + h * g.nsplit * 2 + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                valid = valid && static_cast<uint32_t>(lo >> 32) == g.epoch && static_cast<uint32_t>(hi >> 32) == g.epoch;
+                                mm2[h] = -__uint_as_float(static_cast<uint32_t>(lo));
+                                mm2[HPB + h] = __uint_as_float(static_cast<uint32_t>(hi));
+                            }
+                            ok = __builtin_amdgcn_ballot_w64(!valid) == 0;
+                            if (!ok) __builtin_amdgcn_s_sleep(2);
+                        }
+                        wave_reduce_n<2 * HPB>(mm2, OpMax(), -INFINITY);
+                        if (lane == 0) {
+#pragma unroll
+                            for (int i = 0; i < 2 * HPB; ++i) fold[i] = mm2[i];
+                            *flag = ok ? 1 : 0;
+                            if (!ok && g.status) __hip_atomic_store(g.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                        }
+                    }
+                    __syncthreads();
+                    if (!*flag) return;
+#pragma unroll
+                    for (int h = 0; h < HPB; ++h) { mn[h] = -fold[h]; mx[h] = fold[HPB + h]; }
+                } else {
+                // one fold for both: max of (-min, max) over the chunks
                 float mm2[2 * HPB];
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) {
@@ -932,6 +1022,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                 wave_reduce_n<2 * HPB>(mm2, OpMax(), -INFINITY);
 #pragma unroll
                 for (int h = 0; h < HPB; ++h) { mn[h] = -mm2[h]; mx[h] = mm2[HPB + h]; }
+                }
             }
             float slope[HPB], tmin[HPB];
 #pragma unroll
@@ -1407,7 +1498,10 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             __builtin_amdgcn_s_waitcnt(0);
             __syncthreads();
             int* last = reinterpret_cast<int*>(red);
-            if (tid == 0) *last = __hip_atomic_fetch_add(g.cnt + unit, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == g.nx - 1;
+            if (tid == 0) {
+                if (g.fused) *last = arrive<__HIP_MEMORY_SCOPE_AGENT>(g.done64 + unit, g.epoch) == static_cast<uint32_t>(g.nx);
+                else *last = __hip_atomic_fetch_add(g.cnt + unit, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == g.nx - 1;
+            }
             __syncthreads();
             if (*last) {
                 // the reader: one acquire drops this compute unit's and this die's cached copies of what other
@@ -1441,10 +1535,28 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                     }
                     store_elem<DT>(g.out, row * kD + d, num / den);
                 }
+                // every other workgroup of the unit is past both counters: leave them empty for a replay of this
+                // very launch (a recorded step comes back with the same epoch)
+                if (g.fused) {
+                    for (int i = tid; i < HPB * g.nsplit * 2; i += kNT)
+                        __hip_atomic_store(g.rec + unit * HPB * g.nsplit * 2 + i, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (tid == 0) __hip_atomic_store(g.done64 + unit, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
             }
         }
     }
 }
+
+// ---- the chunked step in one launch: host side ------------------------------------------------------
+// A word of pinned host memory per device that a workgroup sets when it gives up waiting for the other
+// chunks of its unit (allocated once, at the first such call on the device; never freed).  The next chunked
+// call on that device finds it set, reports CQ_ERR_LAUNCH once and the process goes on with two launches.
+constexpr int kMaxDevices = 64;
+static std::atomic<int*> g_status[kMaxDevices];
+static std::atomic<bool> g_fused_off{false};      // set by a give-up; cleared by cq_decode_attn_wait_polls
+static std::atomic<bool> g_fused_wanted{true};    // cq_decode_attn_single_launch
+static std::atomic<uint32_t> g_epoch{0x5eed0000u};
+static std::atomic<int> g_spin_limit{1 << 18};   // polls of about a microsecond each
 
 // Compute units of the current device (a partitioned device reports its own share), asked once per
 // process; kDefaultUnits when there is no device to ask (a host that only plans).
@@ -1468,6 +1580,7 @@ static inline int ngroups(int G, int hpb) { return (G + hpb - 1) / hpb; }
 
 struct Plan {
     int hpb, nh, nt, regl, nsplit, chunk, nx, cap, lds;   // hpb: heads an entry is wide; nh: heads a unit serves
+    bool fused;   // chunked step in one launch: every chunk's workgroup fits the device at once
     size_t ws_mm, ws_part, ws_cnt, ws_lgt;   // chunked launch: min / max, partials, counters; logits (optional)
 };
 
@@ -1508,7 +1621,10 @@ static void plan_for(const cq_decode_args* a, Plan* p, int nh = HPB) {
     const size_t rows = static_cast<size_t>(a->B) * a->Hq;
     p->ws_mm = nsplit > 1 ? ((rows * nsplit * 2 * sizeof(float) + 255) / 256 * 256) : 0;
     p->ws_part = nsplit > 1 ? (rows * p->nx * (kD + 2) * sizeof(float) + 255) / 256 * 256 : 0;
-    p->ws_cnt = nsplit > 1 ? (static_cast<size_t>(units) * sizeof(int) + 255) / 256 * 256 : 0;
+    // counters: [unit] partials written (4 or 8 bytes), then the min / max records of the single-launch step
+    p->ws_cnt = nsplit > 1 ? (static_cast<size_t>(units) * sizeof(unsigned long long) + 255) / 256 * 256 +
+                                 static_cast<size_t>(units) * HPB * nsplit * 16 : 0;
+    p->fused = false;
     // The logits go through a buffer where that is less traffic than the main launch reading the packed K rows
     // again (4 bytes per head and token against the row's 16 or 32 bytes).  Measured at batch 8 x 32 768 tokens,
     // four heads per unit: 2 bits 108.6 -> 90.9 us with the buffer, 1 bit (equal bytes) 52.3 -> 54.0 us.
@@ -1597,6 +1713,15 @@ static int make_plan(const cq_decode_args* a, Plan* p) {
     }
     const int64_t blocks = static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, p->nh) * p->nx;
     if (blocks > 0x7fffffff) return CQ_ERR_SHAPE;
+    // Chunked, and every chunk's workgroup resident at once (two 512-thread workgroups per compute unit, one of
+    // 1024): one launch, the chunks exchange their min / max inside it and keep their logits - no second read of
+    // the packed K rows, no logits buffer.  (The residual units wait for nobody and make room as they end.)
+    if (p->nsplit > 1) {
+        const int64_t waiting = static_cast<int64_t>(a->B) * a->Hkv * ngroups(G, p->nh) * p->nsplit;
+        const int64_t room = static_cast<int64_t>(kPairUnits) * ((p->nt == 512 && p->lds <= kLdsMax / 2) ? 2 : 1);
+        // (one lane per chunk polls)
+        if (waiting <= room && p->nsplit <= 64 && g_fused_wanted.load(std::memory_order_relaxed)) p->fused = true;
+    }
     return CQ_OK;
 }
 
@@ -1634,11 +1759,11 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
     gm.G = G;
     // (a main launch that reads its logits back has no look-up phase for the first workgroup to get ahead in:
     // with the priorities the second one would hold the packed-V loop to itself)
-    gm.ncu = (NT == 512 && !g.lgt && static_cast<int64_t>(units) * g.nx <= 2 * static_cast<int64_t>(pair_units())) ? pair_units() : 0;
+    gm.ncu = (NT == 512 && !g.lgt && !g.fused && static_cast<int64_t>(units) * g.nx <= 2 * static_cast<int64_t>(pair_units())) ? pair_units() : 0;
     gm.d_ng.set(static_cast<uint32_t>(ngroups(G, NH)));
     gm.d_nx.set(static_cast<uint32_t>(g.nx));
     gm.d_hkv.set(static_cast<uint32_t>(g.Hkv));
-    if (g.nsplit > 1) {
+    if (g.nsplit > 1 && !g.fused) {
         DecodeGeom g1 = gm;
         g1.nx = g.nsplit;  // the min/max pass has no residual unit
         g1.d_nx.set(static_cast<uint32_t>(g.nsplit));
@@ -1693,7 +1818,6 @@ constexpr size_t kScratchBytes = static_cast<size_t>(8) << 20;
 // (`used`: no kernel names the array - they get its address as an argument - so nothing else keeps it in the code object)
 static __device__ __align__(256) __attribute__((used)) unsigned char scratch[kScratchBytes];
 
-constexpr int kMaxDevices = 64;
 static std::atomic<void*> g_scratch_ptr[kMaxDevices];
 
 static int scratch_address(void** out) {
@@ -1708,6 +1832,31 @@ static int scratch_address(void** out) {
     }
     *out = p;
     return CQ_OK;
+}
+
+static int* fused_status_word(hipStream_t st) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    int* p = g_status[dev].load(std::memory_order_acquire);
+    if (p) return p;
+    // not while the stream is being recorded: an allocation would end the recording
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    void* raw = nullptr;
+    if (hipHostMalloc(&raw, 64, hipHostMallocDefault) != hipSuccess || !raw) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    *static_cast<volatile int*>(raw) = 0;
+    int* expected = nullptr;
+    if (!g_status[dev].compare_exchange_strong(expected, static_cast<int*>(raw), std::memory_order_acq_rel)) {
+        (void)hipHostFree(raw);   // another host thread was first
+        return expected;
+    }
+    return static_cast<int*>(raw);
 }
 
 static int decode_entry(const cq_decode_args* a, void* workspace, size_t workspace_bytes, bool static_scratch,
@@ -1728,8 +1877,24 @@ static int decode_entry(const cq_decode_args* a, void* workspace, size_t workspa
     // the logits buffer is the last part of the workspace; the static scratch does without it when it
     // does not fit (the main launch then recomputes the logits)
     const size_t need_min = p.ws_mm + p.ws_part + p.ws_cnt;
-    bool with_logits = p.ws_lgt > 0;
+    // One launch when the plan allows it, the caller's own workspace is used (the static entry point allocates
+    // nothing, not even the status word) and no earlier launch of this process gave up waiting.
+    int* status = nullptr;
+    bool fused = p.fused && !static_scratch && !g_fused_off.load(std::memory_order_relaxed);
+    if (fused) {
+        status = fused_status_word(static_cast<hipStream_t>(stream));
+        if (!status) {
+            fused = false;
+        } else if (*static_cast<volatile int*>(status) != 0) {
+            *static_cast<volatile int*>(status) = 0;
+            g_fused_off.store(true, std::memory_order_relaxed);
+            return CQ_ERR_LAUNCH;   // an earlier single-launch step did not complete: its output is not valid
+        }
+    }
+    bool with_logits = !fused && p.ws_lgt > 0;
     if (static_scratch && need_min + p.ws_lgt > kScratchBytes) with_logits = false;
+    // (a plan for one launch sizes the caller's workspace without the logits buffer)
+    if (!static_scratch && p.fused && workspace_bytes < need_min + p.ws_lgt) with_logits = false;
     const size_t need = need_min + (with_logits ? p.ws_lgt : 0);
     if (static_scratch) {
         if (need > kScratchBytes) return CQ_ERR_SCRATCH_LIMIT;
@@ -1753,6 +1918,18 @@ static int decode_entry(const cq_decode_args* a, void* workspace, size_t workspa
     g.mm = static_cast<float*>(workspace);
     g.part = need ? reinterpret_cast<float*>(static_cast<char*>(workspace) + p.ws_mm) : nullptr;
     g.cnt = need ? reinterpret_cast<int*>(static_cast<char*>(workspace) + p.ws_mm + p.ws_part) : nullptr;
+    {
+        const int G = a->Hq / a->Hkv;
+        const size_t units = static_cast<size_t>(a->B) * a->Hkv * ngroups(G, p.nh);
+        char* c0 = reinterpret_cast<char*>(g.cnt);
+        g.done64 = reinterpret_cast<unsigned long long*>(c0);
+        g.rec = reinterpret_cast<unsigned long long*>(c0 + (units * sizeof(unsigned long long) + 255) / 256 * 256);
+    }
+    g.fused = fused ? 1 : 0;
+    g.status = status;
+    g.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
+    uint32_t ep = g_epoch.fetch_add(1, std::memory_order_relaxed) + 1;
+    g.epoch = ep ? ep : g_epoch.fetch_add(1, std::memory_order_relaxed) + 1;   // 0 marks an empty counter
     g.lgt = with_logits ? reinterpret_cast<float*>(static_cast<char*>(workspace) + need_min) : nullptr;
     g.B = a->B; g.Hq = a->Hq; g.Hkv = a->Hkv; g.T = a->T; g.R = a->R; g.S = a->sprompt_len;
     g.nsplit = p.nsplit; g.chunk = p.chunk; g.nx = p.nx;
@@ -1773,7 +1950,22 @@ extern "C" {
 size_t cq_decode_attn_workspace(const cq_decode_args* args) {
     cq::Plan p;
     if (cq::make_plan(args, &p) != CQ_OK) return 0;
-    return p.ws_mm + p.ws_part + p.ws_cnt + p.ws_lgt;
+    return p.ws_mm + p.ws_part + p.ws_cnt + (p.fused ? 0 : p.ws_lgt);
+}
+
+int cq_decode_attn_single_launch(int enable) {
+    const int before = cq::g_fused_wanted.load(std::memory_order_relaxed) ? 1 : 0;
+    if (enable >= 0) cq::g_fused_wanted.store(enable != 0, std::memory_order_relaxed);
+    return before;
+}
+
+int cq_decode_attn_wait_polls(int polls) {
+    const int before = cq::g_spin_limit.load(std::memory_order_relaxed);
+    if (polls >= 0) {
+        cq::g_spin_limit.store(polls, std::memory_order_relaxed);
+        cq::g_fused_off.store(false, std::memory_order_relaxed);
+    }
+    return before;
 }
 
 int cq_decode_attn_plan(const cq_decode_args* args, cq_decode_plan* plan) {
@@ -1785,7 +1977,7 @@ int cq_decode_attn_plan(const cq_decode_args* args, cq_decode_plan* plan) {
     plan->heads_per_unit = p.nh;
     plan->chunks = p.nsplit;
     plan->chunk_tokens = args->T > 0 ? p.chunk : 0;
-    plan->launches = p.nsplit > 1 ? 2 : 1;
+    plan->launches = (p.nsplit > 1 && !p.fused) ? 2 : 1;
     plan->lds_bytes = p.lds;
     plan->register_logits = p.regl;
     return CQ_OK;

@@ -273,14 +273,34 @@ int cq_decode_attn_static(const cq_decode_args* args, cq_stream_t stream);
 typedef struct cq_decode_plan {
     int threads;          /* threads per workgroup: 1024, or 512 with two workgroups per compute unit */
     int heads_per_unit;   /* query heads served by one workgroup (they share a kv head) */
-    int chunks;           /* token chunks per (batch, kv head, head group); > 1: logits + min/max launch, then the main launch (which also merges) */
+    int chunks;           /* token chunks per (batch, kv head, head group); > 1: the chunks' logit min / max are exchanged
+                           * and their partial results merged - in a launch of their own ahead of the main one (launches == 2),
+                           * or inside a single launch when every chunk's workgroup fits the device at once (launches == 1) */
     int chunk_tokens;     /* packed tokens per chunk */
-    int launches;         /* 1 or 2 */
+    int launches;         /* 1 or 2 (what the plan asks for; see cq_decode_attn_wait_polls for when one becomes two) */
     int lds_bytes;        /* dynamic LDS of the main launch */
     int register_logits;  /* > 0: a thread keeps the logits of up to this many of its tokens in registers (fp32)
                            * and the token slots in LDS hold only exp(.) as fp16; 0: fp32 logits wait in the slots */
 } cq_decode_plan;
 int cq_decode_attn_plan(const cq_decode_args* args, cq_decode_plan* plan);
+
+/* The single-launch chunked step (plan: chunks > 1, launches == 1) makes the workgroups of a unit wait for each
+ * other's logit min / max inside the launch.  That is only sound while they are all resident together, which the
+ * plan works out from the device's compute-unit count; the wait is therefore bounded: after `polls` polls (about a
+ * microsecond each; default 262 144) a workgroup gives up, ends without a result and sets a word of pinned host
+ * memory (64 bytes per device, allocated at the first such call outside a stream capture - the one allocation
+ * this library makes - and kept until the process ends).  The next chunked cq_decode_attn on that device then
+ * returns CQ_ERR_LAUNCH once (the previous step's output is not valid) and the process goes on with two launches
+ * per step.  cq_decode_attn_static always takes two launches.  This call sets the bound (polls >= 0; it also
+ * re-enables the single launch after a give-up) and returns the previous one; polls < 0 only queries.
+ * No counterpart in the reference (its kernels never split the token axis). */
+int cq_decode_attn_wait_polls(int polls);
+/* Process-wide switch for the single-launch chunked step (enable != 0: plans may ask for it, the default;
+ * 0: chunked shapes always take two launches - for a process that shares the GPU's compute units with
+ * other work, e.g. through compute-unit masks the plan cannot see; enable < 0 only queries).  Returns the
+ * previous setting.  cq_decode_attn_plan / cq_decode_attn_workspace follow it: size the workspace after
+ * the last change.  No counterpart in the reference. */
+int cq_decode_attn_single_launch(int enable);
 
 /* ------------------------------------------------------------------------
  * Decode-step glue, one launch per layer and token: the (h gs d) split of

@@ -388,9 +388,19 @@ def test_decode_attn_rejects_bad_arguments(ops):
                         g["kr"], g["vr"])
 
 
+@pytest.fixture
+def two_launches():
+    """Chunked shapes take two launches for the test (the process-wide switch of the single-launch step)."""
+    from calibquant_amd import _lib
+    lib = _lib.load()
+    before = lib.cq_decode_attn_single_launch(0)
+    yield
+    lib.cq_decode_attn_single_launch(before)
+
+
 @pytest.mark.parametrize("case", [(2, 16, 8, 20000, 50, 3, 1), (2, 8, 8, 20000, 0, 0, 1), (1, 32, 8, 20000, 33, 5, 2),
                                   (1, 16, 8, 20000, 33, 0, 2)], ids=lambda c: "-".join(str(x) for x in c))
-def test_decode_attn_chunked_with_the_logits_buffer(ops, case):
+def test_decode_attn_chunked_with_the_logits_buffer(ops, case, two_launches):
     """Chunked launches whose first launch hands the logits to the second through the workspace (a packed K row
     of more bytes than the logits: 2 bits, or fewer than four heads per unit), against the oracle.  (Four-head
     units at 1 bit recompute their logits: `test_long_context_batch_8_kv_32768` and the chunked cases above.)"""
@@ -414,18 +424,23 @@ def test_decode_attn_chunked_with_the_logits_buffer(ops, case):
     assert torch.equal(out, out2)
 
 
+@pytest.mark.parametrize("single", [True, False], ids=["one-launch", "two-launches"])
 @pytest.mark.parametrize("case", [(1, 32, 8, 20000, 40, 3, 1), (8, 32, 8, 12000, 0, 0, 1), (2, 32, 8, 12000, 33, 0, 2)],
                          ids=lambda c: "-".join(str(x) for x in c))
-def test_decode_attn_chunked_launches_replayed_from_a_graph(ops, case):
-    """The two chunked launches (counters cleared by the first, partials merged by the last workgroup of a unit in
-    the second; logits through the workspace or recomputed) recorded into a HIP graph: every replay, with eager
-    work and synchronisations in between, gives the bits of the eager call."""
+def test_decode_attn_chunked_launches_replayed_from_a_graph(ops, case, single, request):
+    """The chunked step - two launches (counters cleared by the first, partials merged by the last workgroup of a
+    unit in the second; logits through the workspace or recomputed), or one launch whose chunks exchange their
+    min / max inside it (the records and counters it leaves are emptied by the merging workgroup, so a replay
+    with the same epoch starts clean) - recorded into a HIP graph: every replay, with eager work and
+    synchronisations in between, gives the bits of the eager call."""
+    if not single:
+        request.getfixturevalue("two_launches")
     B, Hq, Hkv, T, R, S, bits = case
     c = make_case(1, Hq, Hkv, 128, T, max(R, 1), bits, "bf16", seed=700 + T + bits, outlier_kind="student")
     g = {k: torch.cat([v] * B, 0) for k, v in case_to_gpu(c, "bf16").items()}
     call = ops.DecodeCall(g["q"], g["ck"], g["cv"], g["sk"], g["zk"], g["sv"], g["zv"], g["kr"] if R else None,
                           g["vr"] if R else None, sprompt_len=S, bits=bits)
-    assert call.plan()["chunks"] > 1
+    assert call.plan()["chunks"] > 1 and call.plan()["launches"] == (1 if single else 2)
     eager = call.run().clone()
     torch.cuda.synchronize()
     want = O.decode_attention(c["q"], c["ck"], c["cv"], c["sk"], c["zk"], c["sv"], c["zv"],

@@ -1,7 +1,7 @@
 """Robustness of the fused decode kernel's other instantiations against the fp32 dequant-attention
 oracle (1e-2 max-abs, 1e-3 mean-abs beyond the storage rounding of the result, see `_check`): logits of magnitude 50-300 (key outlier channels x100, queries
 x3) through the 2-bit paired launch, the 1024-thread launch that keeps a long chunk's logits in
-registers, both hand-over modes of the chunked step and per-token values; and softmax weights built so
+registers, the chunked step in one launch and in two (both hand-over modes) and per-token values; and softmax weights built so
 that the packed-fp16 partial sums of the value loop sit next to 1.0."""
 import numpy as np
 import pytest
@@ -55,8 +55,10 @@ def _large_logit_case(B, Hq, Hkv, T, R, bits, mult, qscale, seed, token_values=F
 LARGE = {
     "2bit-paired": (2, 20, 32, 8, 3328, 128, 2, False, dict(threads=512, chunks=1)),
     "26b-register-logits": (1, 16, 48, 8, 9984, 64, 1, False, dict(threads=1024, chunks=1, register_logits=10)),
-    "chunked-recompute": (1, 8, 32, 8, 20000, 70, 1, False, dict(launches=2)),
-    "chunked-logits-buffer": (1, 8, 32, 8, 12000, 70, 2, False, dict(launches=2)),
+    "chunked-one-launch": (1, 8, 32, 8, 20000, 70, 1, False, dict(launches=1)),
+    "chunked-one-launch-2bit": (1, 8, 32, 8, 12000, 70, 2, False, dict(launches=1)),
+    "chunked-recompute": (1, 12, 32, 8, 20000, 70, 1, False, dict(launches=2)),       # 96 units x 6 chunks: too many to wait
+    "chunked-logits-buffer": (1, 12, 32, 8, 20000, 70, 2, False, dict(launches=2)),
     "token-values": (2, 20, 32, 8, 3328, 128, 1, True, dict(chunks=1)),
     "token-values-2bit": (1, 8, 32, 8, 2000, 40, 2, True, dict(chunks=1)),
 }
@@ -74,6 +76,8 @@ def test_large_logits(ops, name, mult, qscale):
     plan = call.plan()
     for key, val in plan_want.items():
         assert plan[key] == val, (key, plan)
+    if name.startswith("chunked"):
+        assert plan["chunks"] > 1
     out = call.run()
     torch.cuda.synchronize()
     assert torch.equal(out, out[:rows].repeat(reps, 1, 1))
@@ -119,3 +123,36 @@ def test_value_sums_next_to_one(ops, reps, T):
     want = O.decode_attention(c["q"], ck, cv, c["sk"], c["zk"], c["sv"], c["zv"], None, None, 0, 1)
     # the weights are what the case was built for: 1 for the picked tokens, about 2.3e-4 (x the head's factor) elsewhere
     _check(to_np(out[:B]), want)
+
+
+def test_single_launch_chunked_step_gives_up_and_the_host_reports_it(ops):
+    """The wait inside the single-launch chunked step is bounded.  With the bound set to zero polls every
+    workgroup gives up at once (each kernel still ends normally, nothing hangs): the call that launched it
+    returns success, the next chunked call on the device reports CQ_ERR_LAUNCH once, and from then on the
+    process takes two launches - with results equal to the oracle - until the bound is set again."""
+    from calibquant_amd import _lib
+    from tests.util import make_case
+    lib = _lib.load()
+    B, Hq, Hkv, T, R = 2, 32, 8, 20000, 40
+    c = make_case(B, Hq, Hkv, 128, T, R, 1, "bf16", seed=901, outlier_kind="student")
+    g = case_to_gpu(c, "bf16")
+    want = O.decode_attention(c["q"], c["ck"], c["cv"], c["sk"], c["zk"], c["sv"], c["zv"], c["kr"], c["vr"], 0, 1)
+    call = ops.DecodeCall(g["q"], g["ck"], g["cv"], g["sk"], g["zk"], g["sv"], g["zv"], g["kr"], g["vr"], bits=1)
+    assert call.plan()["chunks"] > 1 and call.plan()["launches"] == 1
+    good = call.run().clone()
+    torch.cuda.synchronize()
+    _check(to_np(good), want)
+    before = lib.cq_decode_attn_wait_polls(0)
+    try:
+        call.run()                       # launched; its workgroups give up
+        torch.cuda.synchronize()
+        with pytest.raises(_lib.CalibQuantError):
+            call.run()                   # the host finds the word set
+        out = call.run().clone()         # two launches from here on
+        torch.cuda.synchronize()
+        _check(to_np(out), want)
+    finally:
+        lib.cq_decode_attn_wait_polls(before)      # also re-enables the single launch
+    again = call.run().clone()
+    torch.cuda.synchronize()
+    assert torch.equal(again, good)

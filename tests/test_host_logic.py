@@ -28,7 +28,8 @@ def test_library_loads_and_exports_every_declared_symbol():
 def test_decode_launch_plan_is_a_function_of_the_shape():
     """`cq_decode_attn_plan` (host only): which launch a shape gets.  Two 512-thread workgroups per compute
     unit need a layout within half of the 160 KB LDS and more units of work than the 256 compute units;
-    logits kept in registers only at 1 bit with four heads per unit; chunked shapes take two launches."""
+    logits kept in registers only at 1 bit with four heads per unit; chunked shapes take two launches, or one
+    when all their workgroups fit the device at once."""
     from calibquant_amd import _lib
     lib = _lib.load()
 
@@ -51,9 +52,15 @@ def test_decode_launch_plan_is_a_function_of_the_shape():
     assert plan(64, 32, 8, 3328, 128, force_splits=2) == dict(plan(64, 32, 8, 3328, 128, force_splits=2), threads=1024, launches=2)
     two = plan(128, 16, 8, 3328, 128)                        # two heads per unit: paired, fp32 logits
     assert (two["threads"], two["heads_per_unit"], two["register_logits"]) == (512, 2, 0)
-    long = plan(8, 32, 8, 32768, 0)                          # chunked: the chunks are the units
-    assert long["launches"] == 2 and long["threads"] == 512 and long["chunks"] * long["chunk_tokens"] >= 32768
+    long = plan(8, 32, 8, 32768, 0)                          # chunked: the chunks are the units; all 512 resident: one launch
+    assert long["launches"] == 1 and long["threads"] == 512 and long["chunks"] * long["chunk_tokens"] >= 32768
     assert long["lds_bytes"] <= 80 * 1024
+    assert plan(16, 32, 8, 32768, 0)["launches"] == 2        # twice the workgroups: they cannot all wait for each other
+    assert lib.cq_decode_attn_single_launch(0) == 1          # the process-wide switch
+    try:
+        assert plan(8, 32, 8, 32768, 0) == dict(long, launches=2)
+    finally:
+        assert lib.cq_decode_attn_single_launch(1) == 0
     big = plan(16, 48, 8, 9984, 64)     # six heads per kv head: two exact units of three; one launch
     assert (big["threads"], big["heads_per_unit"], big["launches"], big["register_logits"]) == (1024, 3, 1, 10)   # logits in registers
     assert plan(64, 48, 8, 3328, 128)["heads_per_unit"] == 3 and plan(64, 48, 8, 3328, 128)["threads"] == 512
@@ -95,7 +102,10 @@ def test_decode_launch_plan_invariants_over_random_shapes():
         assert p.chunks >= 1 and p.chunks * p.chunk_tokens >= a.T, shape
         assert p.chunk_tokens % 64 == 0, shape
         assert p.register_logits == 0 or p.chunk_tokens <= p.register_logits * p.threads, shape
-        assert p.launches == (2 if p.chunks > 1 else 1), shape
+        assert p.launches in (1, 2) and (p.launches == 1 or p.chunks > 1), shape
+        if p.launches == 1 and p.chunks > 1:      # one launch: every chunk's workgroup resident at once
+            units_ = a.B * a.Hkv * -(-G_ // p.heads_per_unit)
+            assert units_ * p.chunks <= 256 * (2 if p.threads == 512 else 1) and p.chunks <= 64, shape
         assert (lib.cq_decode_attn_workspace(ctypes.byref(a)) > 0) == (p.chunks > 1), shape
         if a.v_mode == 1:
             assert p.threads == 1024 and p.register_logits == 0, shape

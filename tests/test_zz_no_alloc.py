@@ -68,16 +68,31 @@ def test_static_scratch_entry_point_two_calls_in_a_row():
     g = case_to_gpu(c, "bf16")
     out_ws = torch.zeros((B, Hq, 128), dtype=torch.bfloat16, device="cuda")
     out_st = torch.zeros_like(out_ws)
-    a = _args(_lib, g, B, Hq, Hkv, T, R, S, 2, out_ws)
-    need = lib.cq_decode_attn_workspace(C.byref(a))
-    assert need > lib.cq_decode_attn_static_limit()
-    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
-    a.workspace, a.workspace_bytes = ws.data_ptr(), need
-    assert lib.cq_decode_attn(C.byref(a), stream) == 0
+    single = lib.cq_decode_attn_single_launch(0)      # (two launches for the workspace entry point as well)
+    try:
+        a = _args(_lib, g, B, Hq, Hkv, T, R, S, 2, out_ws)
+        need = lib.cq_decode_attn_workspace(C.byref(a))
+        assert need > lib.cq_decode_attn_static_limit()
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        a.workspace, a.workspace_bytes = ws.data_ptr(), need
+        assert lib.cq_decode_attn(C.byref(a), stream) == 0
+    finally:
+        lib.cq_decode_attn_single_launch(single)
     b = _args(_lib, g, B, Hq, Hkv, T, R, S, 2, out_st)
     assert lib.cq_decode_attn_static(C.byref(b), stream) == 0
     torch.cuda.synchronize()
     assert torch.equal(out_ws, out_st)
+    # ... and the workspace entry point's single launch (the chunks exchange their min / max inside it and
+    # keep their logits: a small workspace) gives the same bits again
+    out_one = torch.zeros_like(out_ws)
+    a = _args(_lib, g, B, Hq, Hkv, T, R, S, 2, out_one)
+    need = lib.cq_decode_attn_workspace(C.byref(a))
+    assert 0 < need < lib.cq_decode_attn_static_limit()
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    a.workspace, a.workspace_bytes = ws.data_ptr(), need
+    assert lib.cq_decode_attn(C.byref(a), stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out_one, out_st)
     want = O.decode_attention(c["q"], c["ck"], c["cv"], c["sk"], c["zk"], c["sv"], c["zv"], c["kr"], c["vr"], S, 2)
     err = np.abs(to_np(out_st) - want)
     assert err.max() < 1e-2 and err.mean() < 1e-3, (T, float(err.max()), float(err.mean()))
