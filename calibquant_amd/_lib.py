@@ -14,7 +14,7 @@ CQ_BF16, CQ_FP16, CQ_FP32, CQ_I64, CQ_I32, CQ_U8 = range(6)
 
 SYMBOLS = (
     "cq_version", "cq_strerror", "cq_last_hip_error",
-    "cq_quantize_pack_workspace", "cq_quantize_pack", "cq_rope_quantize_pack", "cq_rope_rows", "cq_quant", "cq_quant_tensor", "cq_encode",
+    "cq_quantize_pack_workspace", "cq_quantize_pack", "cq_rope_quantize_pack", "cq_rope_rows", "cq_rope_rows_grouped", "cq_quant", "cq_quant_tensor", "cq_encode",
     "cq_lut_vecmat_qk", "cq_lut_vecmat_pv",
     "cq_decode_attn_workspace", "cq_decode_attn", "cq_decode_attn_static", "cq_decode_attn_static_limit",
     "cq_decode_attn_plan", "cq_decode_attn_wait_polls", "cq_decode_attn_single_launch", "cq_rope_append", "cq_quantize_pack_token",
@@ -82,6 +82,9 @@ def load() -> C.CDLL:
     lib.cq_rope_quantize_pack.argtypes = rope_common + [i, f, vp, vp, vp, vp, sz, vp]
     lib.cq_rope_rows.restype = i
     lib.cq_rope_rows.argtypes = rope_common + [vp]
+    lib.cq_rope_rows_grouped.restype = i
+    lib.cq_rope_rows_grouped.argtypes = [vp, i, i, i, i, i, i, i64, i64, i64, i64, vp, vp, i64, vp, i64, i64, i64,
+                                         vp, i64, i64, i64, i64, vp]
     lib.cq_quant_tensor.restype = i
     lib.cq_quant_tensor.argtypes = qargs
     lib.cq_encode.restype = i

@@ -714,6 +714,11 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
         // 32 768 - the rows of the 512 workgroups in flight do not fit the L2s between two passes).
         constexpr bool kKeepRows = MINMAX_ONLY && REGL > 0 && L::KPASS > 1;
         uint4 kall[kKeepRows ? REGL : 1][BITS];
+        // Two table passes in a paired workgroup (2 bits): the first pass requests whole rows and keeps the
+        // 16-byte piece the second pass looks at in registers - requested one piece per pass, every 32-byte row
+        // would cross the memory system twice (a piece is half a row, and memory is fetched by the row or more).
+        constexpr bool kKeepHalf = !MINMAX_ONLY && L::INA && L::KPASS == 2 && BITS == 2 && !kKeepRows;
+        uint4 khalf[kKeepHalf ? REGL : 1];
         auto k_pass = [&](auto pass_c) {
             constexpr int P = decltype(pass_c)::value;
             constexpr int kP0 = (P * L::WPP) / 4;   // first 16-byte piece of a row the pass looks at
@@ -847,6 +852,16 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
 #pragma unroll
                         for (int r = 0; r < L::KR; ++r) {
                             const int tt = min(tb + tid + r * kNT, n - 1);
+                            if constexpr (kKeepHalf) {
+                                static_assert(!kKeepHalf || L::PCS == 1, "a pass looks at one piece of the row");
+                                if constexpr (P == 0) {
+                                    kx[r][0] = ckp[static_cast<int64_t>(tt) * BITS];
+                                    if (ob * L::KR + r < REGL) khalf[ob * L::KR + r] = ckp[static_cast<int64_t>(tt) * BITS + 1];
+                                } else {
+                                    if (ob * L::KR + r < REGL) kx[r][0] = khalf[ob * L::KR + r];
+                                }
+                                continue;
+                            }
 #pragma unroll
                             for (int i = 0; i < L::PCS; ++i) kx[r][i] = ckp[static_cast<int64_t>(tt) * BITS + kP0 + i];
                         }

@@ -425,6 +425,9 @@ struct RopeArgs {
     int64_t pos_sb, pos_st, pos0, table_rows;
     uint16_t* out;            // rotated rows, (B, T, H, 128) through element strides
     int64_t ob, ot, oh;
+    // cq_rope_rows_grouped: every head is a group of `gn` rows, `gs` elements apart in x and `og` in out
+    int gn = 1;
+    int64_t gs = 0, og = 0;
 };
 
 template <typename DT, int BITS, int NR, bool ROPE = false>   // NR: rows per thread (T <= NR * 256)
@@ -917,14 +920,15 @@ template <typename DT>
 __global__ __launch_bounds__(256) void rope_rows_kernel(const uint16_t* __restrict__ x, QuantGeom g, RopeArgs ra) {
     typedef uint32_t U4 __attribute__((ext_vector_type(4)));
     const int64_t gid = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-    const int64_t total = static_cast<int64_t>(g.B) * g.T * g.H * 8;
+    const int64_t total = static_cast<int64_t>(g.B) * g.T * g.H * ra.gn * 8;
     if (gid >= total) return;
     const int p8 = static_cast<int>(gid & 7);
     int64_t r = gid >> 3;
+    const int gq = static_cast<int>(r % ra.gn); r /= ra.gn;
     const int h = static_cast<int>(r % g.H); r /= g.H;
     const int t = static_cast<int>(r % g.T);
     const int b = static_cast<int>(r / g.T);
-    const uint16_t* xr = x + b * g.sb + static_cast<int64_t>(t) * g.st + static_cast<int64_t>(h) * g.sh + p8 * 8;
+    const uint16_t* xr = x + b * g.sb + static_cast<int64_t>(t) * g.st + static_cast<int64_t>(h) * g.sh + gq * ra.gs + p8 * 8;
     int64_t ps = ra.pos ? ra.pos[b * ra.pos_sb + static_cast<int64_t>(t) * ra.pos_st] : ra.pos0 + t;
     ps = ps < 0 ? 0 : (ps >= ra.table_rows ? ra.table_rows - 1 : ps);
     const U4 lo = *reinterpret_cast<const U4*>(xr), hi = *reinterpret_cast<const U4*>(xr + 64);
@@ -941,7 +945,7 @@ __global__ __launch_bounds__(256) void rope_rows_kernel(const uint16_t* __restri
     U4 r1, r2;
 #pragma unroll
     for (int w = 0; w < 4; ++w) { r1[w] = o1[2 * w] | (o1[2 * w + 1] << 16); r2[w] = o2[2 * w] | (o2[2 * w + 1] << 16); }
-    uint16_t* orow = ra.out + b * ra.ob + static_cast<int64_t>(t) * ra.ot + static_cast<int64_t>(h) * ra.oh + p8 * 8;
+    uint16_t* orow = ra.out + b * ra.ob + static_cast<int64_t>(t) * ra.ot + static_cast<int64_t>(h) * ra.oh + gq * ra.og + p8 * 8;
     *reinterpret_cast<U4*>(orow) = r1;
     *reinterpret_cast<U4*>(orow + 64) = r2;
 }
@@ -1141,19 +1145,31 @@ int cq_rope_rows(const void* x, int dtype, int B, int T, int H, int D, int64_t s
                  int64_t stride_h, const void* cos_table, const void* sin_table, int64_t table_rows,
                  const int64_t* pos, int64_t pos_stride_b, int64_t pos_stride_t, int64_t pos0,
                  void* x_rot, int64_t rot_stride_b, int64_t rot_stride_t, int64_t rot_stride_h, cq_stream_t stream) {
+    return cq_rope_rows_grouped(x, dtype, B, T, H, 1, D, stride_b, stride_t, stride_h, 0, cos_table, sin_table, table_rows,
+                                pos, pos_stride_b, pos_stride_t, pos0, x_rot, rot_stride_b, rot_stride_t, rot_stride_h, 0,
+                                stream);
+}
+
+int cq_rope_rows_grouped(const void* x, int dtype, int B, int T, int H, int G, int D, int64_t stride_b, int64_t stride_t,
+                         int64_t stride_h, int64_t stride_g, const void* cos_table, const void* sin_table,
+                         int64_t table_rows, const int64_t* pos, int64_t pos_stride_b, int64_t pos_stride_t, int64_t pos0,
+                         void* x_rot, int64_t rot_stride_b, int64_t rot_stride_t, int64_t rot_stride_h,
+                         int64_t rot_stride_g, cq_stream_t stream) {
     if (!x) return CQ_ERR_NULL;
     if (dtype != CQ_BF16 && dtype != CQ_FP16) return CQ_ERR_DTYPE;
-    if (B < 1 || T < 1 || H < 1) return CQ_ERR_SHAPE;
+    if (B < 1 || T < 1 || H < 1 || G < 1) return CQ_ERR_SHAPE;
     int rc = cq::check_rope(cos_table, sin_table, table_rows, pos, x_rot, rot_stride_b, rot_stride_t, rot_stride_h, D);
     if (rc != CQ_OK) return rc;
-    if ((stride_b % 8) || (stride_t % 8) || (stride_h % 8) || !cq::aligned16(x)) return CQ_ERR_ALIGN;
+    if ((stride_b % 8) || (stride_t % 8) || (stride_h % 8) || (stride_g % 8) || (rot_stride_g % 8) || !cq::aligned16(x))
+        return CQ_ERR_ALIGN;
     cq::QuantGeom g = {};
     g.B = B; g.T = T; g.H = H; g.D = D; g.sb = stride_b; g.st = stride_t; g.sh = stride_h;
     cq::RopeArgs ra;
     ra.cos = static_cast<const uint16_t*>(cos_table); ra.sin = static_cast<const uint16_t*>(sin_table);
     ra.pos = pos; ra.pos_sb = pos_stride_b; ra.pos_st = pos_stride_t; ra.pos0 = pos0; ra.table_rows = table_rows;
     ra.out = static_cast<uint16_t*>(x_rot); ra.ob = rot_stride_b; ra.ot = rot_stride_t; ra.oh = rot_stride_h;
-    const int64_t total = static_cast<int64_t>(B) * T * H * 8;
+    ra.gn = G; ra.gs = stride_g; ra.og = rot_stride_g;
+    const int64_t total = static_cast<int64_t>(B) * T * H * G * 8;
     const int64_t blocks = (total + 255) / 256;
     if (blocks > 0x7fffffff) return CQ_ERR_SHAPE;
     hipStream_t st = static_cast<hipStream_t>(stream);

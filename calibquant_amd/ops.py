@@ -104,6 +104,25 @@ def rope_rows(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, pos, out: O
     return out
 
 
+def rope_rows_grouped(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, pos, out: Optional[torch.Tensor] = None):
+    """`rope_rows` over x (B, T, H, G, D) (any b/t/h/g strides) in one launch: the query block of the fused
+    projection output, where the G query heads of a kv head sit side by side.  `out`: shaped like x."""
+    _need_gpu(x, "x")
+    if x.dim() != 5 or x.stride(4) != 1:
+        raise _lib.CalibQuantError("x must be (B, T, H, G, D) with a contiguous last axis")
+    if out is None:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    if out.shape != x.shape or out.stride(4) != 1:
+        raise _lib.CalibQuantError("rope: out must be shaped like x with a contiguous last axis")
+    args, keep = _rope_args(x[:, :, :, 0], cos, sin, pos, out[:, :, :, 0])
+    (xp, dt, B, T, H, D, sb, st_, sh, cp, sp, rows, pp, psb, pst, p0, op, ob, ot, oh) = args
+    with torch.cuda.device(x.device):
+        rc = _lib.load().cq_rope_rows_grouped(xp, dt, B, T, H, x.shape[3], D, sb, st_, sh, x.stride(3), cp, sp, rows,
+                                              pp, psb, pst, p0, op, ob, ot, oh, out.stride(3), _stream(x))
+    _lib.check(rc, "cq_rope_rows_grouped")
+    return out
+
+
 def rope_quantize_pack(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, pos, out: torch.Tensor,
                        bits: int, clip: float):
     """`quantize_pack(rope(x))` in one pass over x: x (B, T, H, D) is the UN-rotated key block; the

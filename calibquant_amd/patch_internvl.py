@@ -196,8 +196,7 @@ def forward_internlm2_calibquant(self, hidden_states: torch.Tensor, attention_ma
     if hip_rope:
         cos, sin = cos.contiguous(), sin.contiguous()
         q_rot = torch.empty((bsz, q_len, Hkv, G, D), dtype=qkv.dtype, device=qkv.device)
-        for gq in range(G):     # one launch per query head of a group: each is a (B, q, Hkv, D) view of the projection
-            ops.rope_rows(qkv[..., gq, :], cos, sin, position_ids, out=q_rot[..., gq, :])
+        ops.rope_rows_grouped(qkv[..., :G, :], cos, sin, position_ids, out=q_rot)   # all query heads: one launch
         query_states = q_rot.view(bsz, q_len, Hq, D).transpose(1, 2)               # (B, Hq, q, D)
         k_raw = qkv[..., -2, :]                                                    # (B, q, Hkv, D), un-rotated
         k_rot = torch.empty((bsz, q_len, Hkv, D), dtype=qkv.dtype, device=qkv.device)

@@ -105,6 +105,15 @@ int cq_rope_rows(const void* x, int dtype, int B, int T, int H, int D,
                  const int64_t* pos, int64_t pos_stride_b, int64_t pos_stride_t, int64_t pos0,
                  void* x_rot, int64_t rot_stride_b, int64_t rot_stride_t, int64_t rot_stride_h,
                  cq_stream_t stream);
+/* The same over x (B, T, H, G, 128): every head a group of G rows `stride_g` elements apart
+ * (`rot_stride_g` in x_rot) - the query block of the fused projection output, (h gs d) with the
+ * G query heads of a kv head side by side (patch_internvl.py:219-234), in one launch. */
+int cq_rope_rows_grouped(const void* x, int dtype, int B, int T, int H, int G, int D,
+                         int64_t stride_b, int64_t stride_t, int64_t stride_h, int64_t stride_g,
+                         const void* cos_table, const void* sin_table, int64_t table_rows,
+                         const int64_t* pos, int64_t pos_stride_b, int64_t pos_stride_t, int64_t pos0,
+                         void* x_rot, int64_t rot_stride_b, int64_t rot_stride_t, int64_t rot_stride_h,
+                         int64_t rot_stride_g, cq_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * Per-token value quantiser: the reference's

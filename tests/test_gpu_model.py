@@ -65,6 +65,65 @@ def test_patched_forward_decode_matches_oracle_on_one_layer():
         assert err.max().item() < 2e-2 and err.mean().item() < 2e-3
 
 
+def test_masked_steady_state_decode_of_a_left_padded_batch():
+    """A batch whose second sample is left-padded by four positions: prefill with the (B, kv) padding mask,
+    then eight decode steps that each pass the additive (B, 1, 1, kv) mask the reference adds per step
+    (patch_internvl.py:404-410).  Every step's attention output equals wo(oracle attention with that mask) on
+    the module's own packed state and window; the step times with and without the mask are printed (a masked
+    step cannot take the prepared-call fast path: its call object is rebuilt every step)."""
+    import time
+    from calibquant_amd import patch_internvl as pi
+    from calibquant_amd.internlm2 import InternLM2Attention, InternLM2Config
+    torch.manual_seed(7)
+    cfg = InternLM2Config.tiny()
+    B, S, T, TXT, PAD, STEPS = 2, 5, 200, 11, 4, 8
+    N = S + T + TXT
+    lo = torch.finfo(torch.bfloat16).min
+
+    def run(masked):
+        torch.manual_seed(8)
+        att = InternLM2Attention(cfg).cuda().to(torch.bfloat16)
+        att.cq_sprompt_len, att.cq_image_token_num = S, T
+        x = torch.randn(B, N, cfg.hidden_size, device="cuda", dtype=torch.bfloat16)
+        pos = torch.arange(N, device="cuda")[None].expand(B, N).clone()
+        pad = None
+        if masked:
+            pad = torch.ones(B, N, device="cuda", dtype=torch.bool)
+            pad[1, :PAD] = False
+            pos[1] = (pos[1] - PAD).clamp_(min=0)
+        outs, times = [], []
+        with torch.no_grad():
+            _, _, past = pi.forward_internlm2_calibquant(att, x, pad, pos, None, False, True)
+            ck, cv = att.encoded_features_k.cpu().numpy(), att.encoded_features_v.cpu().numpy()
+            sk, zk, sv, zv = (to_np(t) for t in att._cq_stats)
+            for i in range(STEPS):
+                xd = torch.randn(B, 1, cfg.hidden_size, device="cuda", dtype=torch.bfloat16)
+                posd = pos[:, -1:] + 1 + i
+                mask = None
+                if masked:
+                    mask = torch.zeros(B, 1, 1, N + 1 + i, device="cuda", dtype=torch.bfloat16)
+                    mask[1, 0, 0, :PAD] = lo
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                out_d, _, past = pi.forward_internlm2_calibquant(att, xd, mask, posd, past, False, True)
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t0)
+                qd, kd, vd = att.split_qkv(xd)
+                cos, sin = att.rotary_emb(vd, seq_len=N + 1 + i)
+                qd, _ = pi.apply_rotary_pos_emb(qd.transpose(1, 2), kd.transpose(1, 2), cos, sin, posd)
+                m = None if mask is None else to_np(mask[:, 0, 0])
+                want = O.decode_attention(to_np(qd[:, :, 0]), ck, cv, sk, zk, sv, zv, to_np(past[0]), to_np(past[1]), S, 1, mask=m)
+                ref = att.wo(torch.from_numpy(want).cuda().to(torch.bfloat16).reshape(B, 1, -1))
+                err = (out_d.float() - ref.float()).abs()
+                assert err.max().item() < 2e-2 and err.mean().item() < 2e-3, (masked, i, err.max().item())
+                outs.append(out_d)
+        return outs, sorted(times)[len(times) // 2]
+
+    _, t_mask = run(True)
+    _, t_plain = run(False)
+    print(f"\nmasked decode step {t_mask * 1e6:.0f} us, unmasked {t_plain * 1e6:.0f} us per layer (host-inclusive, tiny layer)")
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_fused_decode_step_equals_the_unfused_op_chain(dtype):
     """Several decode steps through the one-launch split + rotary + append path - once driven by the host

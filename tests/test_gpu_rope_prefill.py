@@ -97,6 +97,25 @@ def test_rope_quantize_pack_full_size_equals_the_two_step_path(ops):
     assert torch.equal(rows, _torch_rope(proj[:2, :, :2, -2, :], cos, sin, ar))
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+def test_rope_rows_grouped_equals_one_launch_per_query_head(ops, dtype):
+    """All G query heads of every kv head of a fused projection output in one launch: the bits of the
+    per-head launches (which are pinned to the oracle and to torch's op sequence above)."""
+    B, N, Hkv, G, D = 2, 77, 4, 6, 128
+    k, _ = O.synth_kv(B, N, Hkv * (G + 2), D, dtype, seed=5, outlier_kind="student")
+    proj = to_gpu(k, dtype).view(B, N, Hkv, G + 2, D)
+    cos, sin = _tables(N + 100, D, dtype)
+    pos = (torch.arange(N, device="cuda")[None] + torch.tensor([[0], [57]], device="cuda")).contiguous()
+    out = torch.zeros(B, N, Hkv, G, D, device="cuda", dtype=TDT[dtype])
+    got = ops.rope_rows_grouped(proj[..., :G, :], cos, sin, pos, out=out)
+    torch.cuda.synchronize()
+    assert got is out
+    for gq in range(G):
+        assert torch.equal(out[..., gq, :], ops.rope_rows(proj[..., gq, :], cos, sin, pos))
+    assert torch.equal(ops.rope_rows_grouped(proj[..., :G, :], cos, sin, 3), torch.stack(
+        [ops.rope_rows(proj[..., gq, :], cos, sin, 3) for gq in range(G)], dim=3))
+
+
 def test_rope_quantize_pack_refuses_what_the_one_pass_kernel_cannot_hold(ops):
     from calibquant_amd._lib import CalibQuantError
     x = torch.randn(1, 4000, 2, 128, device="cuda", dtype=torch.bfloat16)
