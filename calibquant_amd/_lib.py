@@ -8,7 +8,9 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libcalibquant_hip.so")
+# CALIBQUANT_HIP_LIBRARY: another build of the same C ABI (the profiling build with phase stops,
+# `python -m calibquant_amd.build --phase-stops`); default: the library built in-tree
+LIB_PATH = os.environ.get("CALIBQUANT_HIP_LIBRARY") or os.path.join(_HERE, "lib", "libcalibquant_hip.so")
 
 CQ_BF16, CQ_FP16, CQ_FP32, CQ_I64, CQ_I32, CQ_U8 = range(6)
 

@@ -94,7 +94,38 @@ def _drain(procs):
             raise RuntimeError(f"hipcc failed on {src}")
 
 
+PHASES_LIBPATH = os.path.join(LIBDIR, "libcalibquant_hip_phases.so")
+
+
+def build_phase_stops(verbose: bool = True) -> str:
+    """The profiling build of the decode source (`-DCQ_PHASE_STOPS`: only the headline instantiation, with
+    early-exit points at the phase boundaries selected by the environment variable CQ_DECODE_PHASE_STOP)
+    as a library of its own, `lib/libcalibquant_hip_phases.so`; `CALIBQUANT_HIP_LIBRARY` makes
+    `calibquant_amd._lib` load it instead of the shipped one.  Used for the per-phase instruction counts
+    under profiles/."""
+    os.makedirs(LIBDIR, exist_ok=True)
+    objs = []
+    for src in SOURCES:
+        obj = os.path.join(LIBDIR, src.replace(".hip", ".phases.o" if src == "cq_decode.hip" else ".o"))
+        if src == "cq_decode.hip" or not os.path.exists(obj):
+            extra = EXTRA_FLAGS.get(src, []) + (["-DCQ_PHASE_STOPS"] if src == "cq_decode.hip" else [])
+            cmd = [HIPCC, *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+            if verbose:
+                print(" ".join(cmd), flush=True)
+            p = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+            _drain([(src, p)])
+        objs.append(obj)
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", PHASES_LIBPATH, *objs]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    return PHASES_LIBPATH
+
+
 if __name__ == "__main__":
+    if "--phase-stops" in sys.argv[1:]:
+        print(build_phase_stops())
+        sys.exit(0)
     print(build())
     print(build_torch_shim())
     sys.exit(0)

@@ -45,6 +45,7 @@
 #endif
 
 #include <atomic>
+#include <cstdlib>
 #include <type_traits>
 
 namespace cq {
@@ -57,6 +58,16 @@ constexpr int kRegPair = 8;        // rounds of logits a thread of a 512-thread 
 constexpr int kRegTwoBit = 4;      // ... of the 2-bit kernel with four heads per unit (4 096 tokens)
 constexpr int kRegLong = 10;       // ... of a 1024-thread workgroup that holds a long chunk in one launch (10 240 tokens)
 constexpr float kLog2e = 1.4426950408889634f;
+
+// Profiling build (-DCQ_PHASE_STOPS, `python -m calibquant_amd.build --phase-stops`; only the headline
+// instantiation is compiled): a launch can be told to end at a phase boundary (environment variable
+// CQ_DECODE_PHASE_STOP = k, read per call), so that whole-launch hardware counters of runs with successive
+// k give per-phase counts by subtraction.  The shipped library has none of this.
+#ifdef CQ_PHASE_STOPS
+#define CQ_PHASE(k) do { if (g.stop == (k)) return; } while (0)
+#else
+#define CQ_PHASE(k) do { } while (0)
+#endif
 
 
 template <int N> struct alignas(N * 4) Vec { float v[N]; };
@@ -93,6 +104,9 @@ struct DecodeGeom {
     uint32_t epoch;
     int fused;
     int spin_limit;
+#ifdef CQ_PHASE_STOPS
+    int stop;     // phase boundary at which the launch ends (-1: runs to the end)
+#endif
     int B, Hq, Hkv, T, R, S;
     int nsplit, chunk, nx;
     int calib;
@@ -453,6 +467,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
         }
     };
 
+    CQ_PHASE(1);   // prologue, requests of q and the statistics
     // ---- phase 0: q, per-bit weights ---------------------------------------------------
     if (tid < HPB * kD) {
         const int h = tid / kD, d = tid % kD;
@@ -567,6 +582,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
         for (int r = kVEarly; r < kPF; ++r) request_v(r);
         if constexpr (REGL == 0) for_my_tokens(n, [&](int rd, int tt) { store_logits(rd, tt, gl[tt]); });
     }
+    CQ_PHASE(2);   // q, per-bit weights, first packed K rows requested
     if (k_rows) {
         // ---- phase 2: byte table = high-nibble table + low-nibble table ----------------
         // nibble tables: entry (j, half, v) = sum of the per-bit weights v selects; the
@@ -895,6 +911,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             k_pass(std::integral_constant<int, 3>{});
         }
     }
+    CQ_PHASE(3);   // K table and look-ups
     phase_priority(std::integral_constant<int, 2>{});
     if (k_rows) {   // one reduction for both: max of (-min, max)
         float mm2[2 * HPB];
@@ -905,6 +922,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
         for (int h = 0; h < HPB; ++h) { mn[h] = -mm2[h]; mx[h] = mm2[HPB + h]; }
     }
 
+    CQ_PHASE(4);   // block min / max
     if constexpr (MINMAX_ONLY) {
 #pragma unroll
         for (int h = 0; h < HPB; ++h) {
@@ -981,6 +999,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                 for (int r = 0; r < kPF; ++r) vc[r] = cvp4[min((vs0 + tid + (r / BITS) * kNT) * BITS + r % BITS, last_u)];
             };
 
+            CQ_PHASE(5);   // staging of the first packed V block
             // ---- phase 4: calibration + exp ---------------------------------------------
             if constexpr (CHUNKED) {
                 if (g.fused) {
@@ -1141,6 +1160,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             // keeps its partial through the packed-V phase and the fold rides on that phase's
             // closing barriers.
             __syncthreads();   // publishes e and vst
+            CQ_PHASE(6);   // calibration and exponentials
             // (requested here, not right after the staging: the logits' registers are free now)
             if constexpr (kVAhead) request_v_block(L::VSUB);
 
@@ -1303,6 +1323,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                     v_flush(s0);
                 }
             }
+            CQ_PHASE(7);   // packed-V loop (tables, look-ups, sums; staging of the later blocks)
             phase_priority(std::integral_constant<int, 4>{});
             load_res_k(0, rk);   // first residual tile's K rows: in flight during the fold below
             // per-wave partial sums of e (and of e * minimum), folded by the output threads below
@@ -1366,6 +1387,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
         }
 
         if (n == 0) load_res_k(0, rk);
+        CQ_PHASE(8);   // fold of the packed part
         // ---- phase 6: full-precision residual rows, online softmax.  Runs last: its first
         // tile is requested when the packed-V phase ends and arrives during that phase's fold.
 #pragma unroll
@@ -1482,6 +1504,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                 if (n == 0) stat[4 * HPB + h] = 0.f;
             }
         }
+        CQ_PHASE(9);   // residual window
         // ---- phase 7: merge / write ---------------------------------------------------------
         __syncthreads();
         if (tid < nh * kD) {
@@ -1795,6 +1818,12 @@ static int launch(const DecodeGeom& g, const Plan& p, hipStream_t st) {
 
 template <typename DT, bool VTOK>
 static int dispatch(const DecodeGeom& g, const Plan& p, int bits, hipStream_t st) {
+#ifdef CQ_PHASE_STOPS
+    if constexpr (!VTOK && std::is_same<DT, BF16>::value) {
+        if (bits == 1 && p.hpb == 4 && p.nh == 4 && p.nt == 512) return launch<1, 4, DT, false, 512, kRegPair>(g, p, st);
+    }
+    return CQ_ERR_UNSUPPORTED;
+#else
     if constexpr (!VTOK) {
         if (p.nh == 3 && p.hpb == 4) {   // exact units of three heads
             if (bits == 1) {
@@ -1822,6 +1851,7 @@ static int dispatch(const DecodeGeom& g, const Plan& p, int bits, hipStream_t st
     }
     if (p.hpb == 2) return launch<2, 2, DT, VTOK>(g, p, st);
     return launch<2, 1, DT, VTOK>(g, p, st);
+#endif
 }
 
 // ---- static scratch for callers that cannot allocate --------------------------------------------
@@ -1940,6 +1970,12 @@ static int decode_entry(const cq_decode_args* a, void* workspace, size_t workspa
         g.done64 = reinterpret_cast<unsigned long long*>(c0);
         g.rec = reinterpret_cast<unsigned long long*>(c0 + (units * sizeof(unsigned long long) + 255) / 256 * 256);
     }
+#ifdef CQ_PHASE_STOPS
+    {
+        const char* e = getenv("CQ_DECODE_PHASE_STOP");
+        g.stop = e ? atoi(e) : -1;
+    }
+#endif
     g.fused = fused ? 1 : 0;
     g.status = status;
     g.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
