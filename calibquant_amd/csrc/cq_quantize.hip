@@ -19,6 +19,8 @@
 // only compares - the per-element IEEE division would otherwise bound the pass.
 #include "cq_common.h"
 
+#include <atomic>
+
 #include <mutex>
 #include <vector>
 
@@ -406,7 +408,7 @@ __global__ __launch_bounds__(kQThreads) void emit_kernel(const uint16_t* __restr
 constexpr int kFThreads = 1024;
 constexpr int kFRows = 13;                  // rows per thread at most (13 x 256 = 12 tiles + thumbnail of 256 tokens)
 constexpr int kFMaxT = kFRows * (kFThreads / 4);
-constexpr int kFGrid = 256;                 // workgroups of the persistent launch (one per compute unit)
+constexpr int kFGridDefault = 256;          // workgroups of the persistent launch when no device can be asked: a whole MI355X
 // rows per thread of the next slice that are staged in LDS (16 KB each for the workgroup)
 // (not with the rotary embedding fused in: that instantiation has no registers to spare for the addresses)
 constexpr int fused_stage_rows(int nr, bool rope) { return (nr > 8 && !rope) ? 8 : 0; }
@@ -803,6 +805,21 @@ static int launch_fused(dim3 grid, hipStream_t st, const uint16_t* xp, const Qua
 }
 
 // true if the shape goes through the one-pass kernel (x read once, slice by slice in registers)
+// Compute units of the current device, asked once per process.
+static int persistent_units() {
+    static std::atomic<int> cached{0};
+    int n = cached.load(std::memory_order_relaxed);
+    if (n > 0) return n;
+    int dev = 0, cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cu < 1) {
+        (void)hipGetLastError();   // not an error of the caller's
+        cu = kFGridDefault;
+    }
+    cached.store(cu, std::memory_order_relaxed);
+    return cu;
+}
+
 static bool one_pass_shape(const QuantGeom& g, const uint8_t* codes) {
     return g.D == 128 && g.T <= kFMaxT && (reinterpret_cast<uintptr_t>(codes) & 3u) == 0 &&
            static_cast<int64_t>(g.B) * g.H < (static_cast<int64_t>(1) << 31) && g.st > 0 && g.st * 2 < (1 << 24) &&
@@ -822,7 +839,11 @@ static int run_quant(const void* x, QuantGeom g, int bits, float clip, uint8_t* 
         const int64_t bh8 = (static_cast<int64_t>(g.B) * g.H + 7) / 8;
         // persistent: at most one workgroup per compute unit and a multiple of 32 of them
         const int64_t nsl = bh8 * 32;
-        const dim3 fgrid(static_cast<unsigned>(nsl < kFGrid ? nsl : kFGrid));
+        // (the compute-unit count of the current device - a partitioned device reports its own share -
+        // rounded down to the multiple of 32 the slice walk needs)
+        const int cu = persistent_units();
+        const int64_t fmax = cu >= 32 ? cu / 32 * 32 : 32;
+        const dim3 fgrid(static_cast<unsigned>(nsl < fmax ? nsl : fmax));
         const int nr = (g.T + kFThreads / 4 - 1) / (kFThreads / 4);
         const RopeArgs ra = rope ? *rope : RopeArgs{};
 #define CQ_FUSED(B_, N_)                                                                          \

@@ -63,7 +63,11 @@ class RMSNorm(nn.Module):
 
     def forward(self, x):
         # one fused normalisation launch (fp32 statistics inside) instead of the six element-wise
-        # launches of the textbook form: at decode the layer is bound by launches on the host
+        # launches of the textbook form: at decode the layer is bound by launches on the host.
+        # (It rounds once, after the multiplication by the weight; the textbook form rounds the normalised
+        # activations to the storage dtype before that multiplication.  The stand-in model's values shift by
+        # that rounding - in its 1-bit and its full-precision runs alike; nothing on the quantised path
+        # depends on it.)
         return F.rms_norm(x, self.weight.shape, self.weight, self.eps)
 
 

@@ -117,8 +117,9 @@ def custom_generate(self, pixel_values=None, input_ids=None, attention_mask=None
 def _image_token_num(self) -> int:
     """The image token count of this forward: the explicit override `cq_image_token_num` on the
     module if a caller set one (`custom_generate` does), else the `IMAGE_TOKEN_NUM` environment
-    variable, re-read on every forward as the reference does (patch_internvl.py:189,251) - a caller
-    that only updates the variable between prompts gets the new count."""
+    variable, re-read on every prefill and on every decode step that does not take the prepared
+    steady-state step (the reference re-reads it per forward, patch_internvl.py:189,251) - a caller
+    that updates the variable between prompts gets the new count with the next prefill."""
     n = getattr(self, "cq_image_token_num", None)
     if n is None:
         env = os.environ.get("IMAGE_TOKEN_NUM")
@@ -140,7 +141,9 @@ def forward_internlm2_calibquant(self, hidden_states: torch.Tensor, attention_ma
     (`encoded_features_k/v`, `scale_key/value`, `zero_point_key/value`, `unique_values_k/v`)."""
     # steady-state decode: the step object the first decode step prepared runs the whole step (rotary
     # embedding + window append launch, attention launch) in one call into the host shim; it declines
-    # (returns None) when this is not the next token of the window it owns
+    # (returns None) when this is not the next token of the window it owns.  The hyper-parameters
+    # (`cq_sprompt_len`, `cq_bits`, `cq_v_mode`, the image token count) are the ones of the first decode
+    # step after a prefill: on this path they are not read again until the next prefill or a decline.
     fast = self.__dict__.get("_cq_step")
     if (fast is not None and attention_mask is None and past_key_value is not None and position_ids is not None
             and not kwargs and hidden_states.shape[1] == 1):

@@ -241,17 +241,25 @@ def _prefill(m, ids, pix=None):
     return lm.forward_step(emb, pos, None)
 
 
-@pytest.mark.parametrize("quantized,fp_kernel", [(True, False), (False, False), (False, True)])
-def test_static_decoder_graph_replays_equal_eager_steps(quantized, fp_kernel):
+@pytest.mark.parametrize("quantized,fp_kernel,width", [(True, False, "tiny"), (False, False, "tiny"), (False, True, "tiny"),
+                                                       (True, False, "26b")])
+def test_static_decoder_graph_replays_equal_eager_steps(quantized, fp_kernel, width):
     """The recorded decode step, replayed per token, produces the tokens of the same step run
-    eagerly, and its first step agrees with the model's own eager step."""
+    eagerly, and its first step agrees with the model's own eager step.  `26b`: two layers of the
+    InternLM2-20B width (hidden 6 144, 48 query / 8 kv heads: units of three heads) at batch 6."""
     from calibquant_amd import patch_internvl as pi
     from calibquant_amd.graph_decode import StaticDecoder
-    from calibquant_amd.internlm2 import InternLM2Attention, InternVLChatStandIn
+    from calibquant_amd.internlm2 import InternLM2Attention, InternLM2Config, InternVLChatStandIn
     fp_forward, fp_generate = InternLM2Attention.forward, InternVLChatStandIn.generate
-    m = _tiny_model(seed=5)
+    if width == "26b":
+        torch.manual_seed(5)
+        cfg = InternLM2Config(vocab_size=512, hidden_size=6144, intermediate_size=16384, num_hidden_layers=2,
+                              num_attention_heads=48, num_key_value_heads=8, max_position_embeddings=8192)
+        m = InternVLChatStandIn(cfg).cuda().to(torch.bfloat16).eval()
+    else:
+        m = _tiny_model(seed=5)
     lm = m.language_model
-    B, S, tiles, txt, NEW = 2, 41, 2, 9, 12
+    B, S, tiles, txt, NEW = (6 if width == "26b" else 2), 41, 2, 9, 12
     T = tiles * 256
     ids = torch.randint(0, 500, (B, S + T + txt), device="cuda")
     ids[:, S:S + T] = m.img_context_token_id

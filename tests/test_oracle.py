@@ -327,7 +327,8 @@ def test_decode_attention_no_image_or_no_residual():
 def test_refchain_is_close_to_fp32_oracle():
     q, ck, cv, sk, zk, sv, zv, kr, vr = _case(T=512, R=32, D=64)
     a = O.decode_attention(q, ck, cv, sk, zk, sv, zv, kr, vr, 8, 1)
-    b = O.decode_attention_refchain(q, ck, cv, sk, zk, sv, zv, kr, vr, 8, 1, "bf16")
+    from tests.refchain import decode_attention_refchain
+    b = decode_attention_refchain(q, ck, cv, sk, zk, sv, zv, kr, vr, 8, 1, "bf16")
     assert np.abs(a - b).max() < 5e-2 and np.abs(a - b).mean() < 1e-2
 
 
@@ -438,3 +439,40 @@ def test_oracle_results_are_frozen_by_the_committed_digests():
             assert g[key] == w[key], (name, key)
         assert np.allclose(g["out_head0"], w["out_head0"], atol=2e-6), name
         assert abs(g["out_sum"] - w["out_sum"]) < 1e-3, name
+
+
+def test_chunk_partials_merge_like_the_unchunked_softmax():
+    """The arithmetic of the chunked step's merge, on the CPU: every chunk leaves (m, l, acc) = (its maximum
+    logit, the sum of exp(w - m), the exp-weighted value sum); combining them eight at a time with a running
+    (m, numerator, denominator) - the order the merging workgroup uses, with chunks that are masked out
+    entirely (m = -inf) and a residual partial among them - gives the softmax-weighted sum over all
+    positions, whatever the chunking."""
+    rng = np.random.default_rng(3)
+    for nchunk, T, D in ((1, 50, 8), (8, 400, 16), (9, 333, 8), (19, 1000, 4)):
+        w = rng.standard_normal(T) * 5
+        w[rng.random(T) < 0.1] = -np.inf
+        v = rng.standard_normal((T, D))
+        bounds = np.linspace(0, T, nchunk + 1).astype(int)
+        if nchunk > 2:
+            w[bounds[1]:bounds[2]] = -np.inf            # a chunk with every position masked
+        parts = []
+        for c in range(nchunk):
+            ws, vs = w[bounds[c]:bounds[c + 1]], v[bounds[c]:bounds[c + 1]]
+            m = ws.max() if ws.size else -np.inf
+            e = np.zeros_like(ws) if m == -np.inf else np.exp(ws - m)
+            parts.append((m, e.sum(), e @ vs))
+        m, num, den = -np.inf, np.zeros(D), 0.0
+        for s0 in range(0, nchunk, 8):
+            blk = parts[s0:s0 + 8]
+            mb = max([m] + [p_[0] for p_ in blk])
+            keep = 0.0 if m == -np.inf else np.exp(m - mb)
+            num, den = num * keep, den * keep
+            for pm, pl, pa in blk:
+                wgt = 0.0 if pm == -np.inf else np.exp(pm - mb)
+                den += pl * wgt
+                num = num + pa * wgt
+            m = mb
+        ok = np.isfinite(w)
+        p_full = np.exp(w[ok] - w[ok].max())
+        want = (p_full / p_full.sum()) @ v[ok]
+        assert np.allclose(num / den, want, rtol=1e-12, atol=1e-12)
