@@ -294,12 +294,12 @@ __device__ __forceinline__ void publish(float* p, float v) {
 }
 
 // One more arrival at an epoch-tagged counter; returns the arrivals of this epoch including this one.
-// SCOPE: device scope (the exchange is done where all dies see it), or workgroup scope, which this hardware
-// executes in the L2 of the issuing die like every read-modify-write - the fast form, for counters that only
-// workgroups of one die touch.
-// The current value of a 64-bit word as the L2 (or, at device scope, the memory side) holds it: a compare-and-
-// swap of 0 for 0.  (Not a read-modify-write that changes nothing, such as OR 0: the compiler turns those into
-// plain loads, which a compute unit's own cache may answer with what it read earlier.)
+// Measured on this device: an atomic read-modify-write is executed at the memory side whatever scope it names
+// (about 2 us a round trip, those on one address one after the other), so such counters are for counting once
+// per workgroup, never for polling.
+// peek64: the current value of a 64-bit word as the memory side holds it, a compare-and-swap of 0 for 0.  (Not a
+// read-modify-write that changes nothing, such as OR 0: the compiler turns those into plain loads, which a
+// compute unit's own cache may answer with what it read earlier.)
 template <int SCOPE>
 __device__ __forceinline__ unsigned long long peek64(unsigned long long* c) {
     unsigned long long v = 0ull;
@@ -316,6 +316,15 @@ __device__ __forceinline__ uint32_t arrive(unsigned long long* c, uint32_t epoch
         if (__hip_atomic_compare_exchange_strong(c, &old, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED, SCOPE))
             return static_cast<uint32_t>(want);
     }
+}
+
+// The single-launch chunked step's records and arrival counter of one unit back to empty: by the unit's last
+// workgroup, once every other one is past both.
+template <int HPB, int NT>
+__device__ __forceinline__ void clear_handover(const DecodeGeom& g, int64_t unit, int tid) {
+    for (int i = tid; i < HPB * g.nsplit * 2; i += NT)
+        __hip_atomic_store(g.rec + unit * HPB * g.nsplit * 2 + i, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) __hip_atomic_store(g.done64 + unit, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __device__ __forceinline__ uint32_t pack_f16(float a, float b) {
@@ -1035,7 +1044,16 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                         }
                     }
                     __syncthreads();
-                    if (!*flag) return;
+                    if (!*flag) {
+                        // Given up: no result from this workgroup, but it is still counted, so that the unit's
+                        // last workgroup - this one or another - leaves the records and the counter empty and a
+                        // replay of this very launch (same epoch) does not take this launch's records for its own.
+                        int* last = reinterpret_cast<int*>(red);
+                        if (tid == 0) *last = arrive<__HIP_MEMORY_SCOPE_AGENT>(g.done64 + unit, g.epoch) == static_cast<uint32_t>(g.nx);
+                        __syncthreads();
+                        if (*last) clear_handover<HPB, kNT>(g, unit, tid);
+                        return;
+                    }
 #pragma unroll
                     for (int h = 0; h < HPB; ++h) { mn[h] = -fold[h]; mx[h] = fold[HPB + h]; }
                 } else {
@@ -1575,11 +1593,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                 }
                 // every other workgroup of the unit is past both counters: leave them empty for a replay of this
                 // very launch (a recorded step comes back with the same epoch)
-                if (g.fused) {
-                    for (int i = tid; i < HPB * g.nsplit * 2; i += kNT)
-                        __hip_atomic_store(g.rec + unit * HPB * g.nsplit * 2 + i, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    if (tid == 0) __hip_atomic_store(g.done64 + unit, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
+                if (g.fused) clear_handover<HPB, kNT>(g, unit, tid);
             }
         }
     }
@@ -2008,6 +2022,14 @@ int cq_decode_attn_single_launch(int enable) {
     const int before = cq::g_fused_wanted.load(std::memory_order_relaxed) ? 1 : 0;
     if (enable >= 0) cq::g_fused_wanted.store(enable != 0, std::memory_order_relaxed);
     return before;
+}
+
+int cq_decode_attn_gave_up(void) {
+    for (int dev = 0; dev < cq::kMaxDevices; ++dev) {
+        const int* p = cq::g_status[dev].load(std::memory_order_acquire);
+        if (p && *static_cast<const volatile int*>(p) != 0) return 1;
+    }
+    return 0;
 }
 
 int cq_decode_attn_wait_polls(int polls) {

@@ -410,8 +410,14 @@ constexpr int kFRows = 13;                  // rows per thread at most (13 x 256
 constexpr int kFMaxT = kFRows * (kFThreads / 4);
 constexpr int kFGridDefault = 256;          // workgroups of the persistent launch when no device can be asked: a whole MI355X
 // rows per thread of the next slice that are staged in LDS (16 KB each for the workgroup)
-// (not with the rotary embedding fused in: that instantiation has no registers to spare for the addresses)
+// (not with the rotary embedding fused in: that instantiation has no registers to spare for the addresses).
+// The staged loads are assembly that the compiler does not see (m0, their own wait count): building with
+// -DCQ_NO_LDS_STAGE refills every row from memory through registers instead, for a toolchain that breaks them.
+#ifdef CQ_NO_LDS_STAGE
+constexpr int fused_stage_rows(int, bool) { return 0; }
+#else
 constexpr int fused_stage_rows(int nr, bool rope) { return (nr > 8 && !rope) ? 8 : 0; }
+#endif
 
 // Rotary embedding fused into the pass (ROPE): x is the un-rotated key block; every row is rotated as it
 // arrives - rnd(rnd(x * cos) + rotate_half(x) * sin), the arithmetic of the ops the reference runs on the

@@ -25,7 +25,7 @@ from typing import List, Optional
 import torch
 import torch.nn.functional as F
 
-from . import ops
+from . import _lib, ops
 from ._lib import CalibQuantError
 from .patch_internvl import CALIB_OFFSET_MAX, CALIB_OFFSET_MIN
 
@@ -167,4 +167,12 @@ class StaticDecoder:
             out.append(self.step().clone())
             if on_step is not None:
                 on_step(i)
-        return torch.stack(out, dim=1)
+        tokens = torch.stack(out, dim=1)
+        # A replayed launch does not pass through the library's own check of the single-launch chunked step's
+        # bounded wait (long contexts only): ask once the replays are done.
+        if self.graph is not None:
+            torch.cuda.synchronize()
+            if _lib.load().cq_decode_attn_gave_up():
+                raise CalibQuantError("a recorded decode step did not complete (single-launch chunked step gave "
+                                           "up waiting); rerun with cq_decode_attn_single_launch(0)")
+        return tokens

@@ -344,7 +344,7 @@ class DecodeCall:
             a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
             keep.append(ws)
         self.args, self._ref, self._keep, self.out, self.device = a, C.byref(a), keep, out, q.device
-        self.workspace_bytes = 0 if ws is None else ws.numel()
+        self.workspace, self.workspace_bytes = ws, 0 if ws is None else ws.numel()
 
     def plan(self) -> dict:
         """What the launch will be for the prepared arguments (`cq_decode_attn_plan`): threads per

@@ -304,6 +304,12 @@ int cq_decode_attn_plan(const cq_decode_args* args, cq_decode_plan* plan);
  * re-enables the single launch after a give-up) and returns the previous one; polls < 0 only queries.
  * No counterpart in the reference (its kernels never split the token axis). */
 int cq_decode_attn_wait_polls(int polls);
+/* 1 while a give-up is flagged on some device and no cq_decode_attn call has reported it yet, else 0; a read
+ * of host memory, no device call.  For callers that replay a recorded single-launch step (a HIP graph) and so
+ * never pass through the check inside cq_decode_attn: ask after synchronising with the replays.  A launch
+ * whose workgroups gave up leaves the workspace as a finished one does, so later replays are not affected by
+ * it.  No counterpart in the reference. */
+int cq_decode_attn_gave_up(void);
 /* Process-wide switch for the single-launch chunked step (enable != 0: plans may ask for it, the default;
  * 0: chunked shapes always take two launches - for a process that shares the GPU's compute units with
  * other work, e.g. through compute-unit masks the plan cannot see; enable < 0 only queries).  Returns the

@@ -127,8 +127,8 @@ def test_value_sums_next_to_one(ops, reps, T):
 
 def test_single_launch_chunked_step_gives_up_and_the_host_reports_it(ops):
     """The wait inside the single-launch chunked step is bounded.  With the bound set to zero polls every
-    workgroup gives up at once (each kernel still ends normally, nothing hangs): the call that launched it
-    returns success, the next chunked call on the device reports CQ_ERR_LAUNCH once, and from then on the
+    workgroup gives up at once (each kernel still ends normally, nothing hangs, and the workspace's hand-over
+    words are left empty as after a finished launch): the call that launched it returns success, the next chunked call on the device reports CQ_ERR_LAUNCH once, and from then on the
     process takes two launches - with results equal to the oracle - until the bound is set again."""
     from calibquant_amd import _lib
     from tests.util import make_case
@@ -142,12 +142,26 @@ def test_single_launch_chunked_step_gives_up_and_the_host_reports_it(ops):
     good = call.run().clone()
     torch.cuda.synchronize()
     _check(to_np(good), want)
+    assert lib.cq_decode_attn_gave_up() == 0
+    # the hand-over words (a counter per unit, then two records per head and chunk) are the tail of the workspace
+    units, heads, chunks = B * Hkv, call.plan()["heads_per_unit"], call.plan()["chunks"]
+    rec = units * heads * chunks * 16
+    cnt = (units * 8 + 255) // 256 * 256 + rec
+
+    def handover_words():
+        return torch.cat([call.workspace[-cnt:][:units * 8], call.workspace[-rec:]])
+    assert not handover_words().any(), "a finished launch leaves its hand-over words empty"
     before = lib.cq_decode_attn_wait_polls(0)
     try:
         call.run()                       # launched; its workgroups give up
         torch.cuda.synchronize()
+        # ... and so does one whose workgroups gave up: a replay of that very launch (a recorded step comes
+        # back with the same epoch) must not find this launch's records
+        assert not handover_words().any()
+        assert lib.cq_decode_attn_gave_up() == 1
         with pytest.raises(_lib.CalibQuantError):
             call.run()                   # the host finds the word set
+        assert lib.cq_decode_attn_gave_up() == 0      # reported
         out = call.run().clone()         # two launches from here on
         torch.cuda.synchronize()
         _check(to_np(out), want)
