@@ -19,7 +19,7 @@ SYMBOLS = (
     "cq_quantize_pack_workspace", "cq_quantize_pack", "cq_rope_quantize_pack", "cq_rope_rows", "cq_rope_rows_grouped", "cq_quant", "cq_quant_tensor", "cq_encode",
     "cq_lut_vecmat_qk", "cq_lut_vecmat_pv",
     "cq_decode_attn_workspace", "cq_decode_attn", "cq_decode_attn_static", "cq_decode_attn_static_limit",
-    "cq_decode_attn_plan", "cq_decode_attn_wait_polls", "cq_decode_attn_gave_up", "cq_decode_attn_single_launch", "cq_rope_append", "cq_quantize_pack_token",
+    "cq_decode_attn_plan", "cq_decode_attn_wait_polls", "cq_decode_attn_gave_up", "cq_quantize_pack_wait_polls", "cq_decode_attn_single_launch", "cq_rope_append", "cq_quantize_pack_token",
 )
 
 
@@ -104,6 +104,8 @@ def load() -> C.CDLL:
     lib.cq_decode_attn.argtypes = [C.POINTER(DecodeArgs), vp]
     lib.cq_decode_attn_wait_polls.restype = i
     lib.cq_decode_attn_wait_polls.argtypes = [i]
+    lib.cq_quantize_pack_wait_polls.restype = i
+    lib.cq_quantize_pack_wait_polls.argtypes = [i]
     lib.cq_decode_attn_gave_up.restype = i
     lib.cq_decode_attn_gave_up.argtypes = []
     lib.cq_decode_attn_single_launch.restype = i

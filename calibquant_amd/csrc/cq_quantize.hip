@@ -38,6 +38,16 @@ struct QuantGeom {
     FastDiv dT, dH;       // divisors T and H of a flat (b, h, t) row index (per-token quantiser)
     FastDiv dTB;          // per-token quantiser: blocks of 16 tokens per (batch, head)
     int shared_stats;     // non-zero: one row of statistics / thresholds serves every (batch, head) (whole-tensor mode)
+    // One-pass kernel on a token axis that is longer than a workgroup's registers hold (SPLIT): 2^parts_log2
+    // workgroups share a slice, `part_rows` rows each, and exchange their channel minima / maxima through `rec`
+    // inside the launch: [virtual slice][channel][2] 64-bit records, the float's bits below the call's epoch, so a
+    // record is valid by itself and nothing has to be cleared.  The wait for the other parts is bounded
+    // (spin_limit polls); a lane that gives up sets *status (pinned host memory).
+    int parts_log2, part_rows;
+    unsigned long long* rec;
+    uint32_t epoch;
+    int spin_limit;
+    int* status;
 };
 
 static inline int pick_chunks(int B, int T, int H) {
@@ -438,7 +448,12 @@ struct RopeArgs {
     int64_t gs = 0, og = 0;
 };
 
-template <typename DT, int BITS, int NR, bool ROPE = false>   // NR: rows per thread (T <= NR * 256)
+// SPLIT: the token axis is longer than NR * 256 rows: 2^g.parts_log2 workgroups share a slice, each with g.part_rows
+// of its rows (<= NR * 256) in registers, and exchange their channels' min / max before the statistics - x is still
+// read once.  The parts of a slice are consecutive ids, i.e. they are worked on by different workgroups of the
+// persistent launch in the same step of their walks (the grid is a multiple of the part count), all of them
+// resident: whoever waits, waits for workgroups that are running.
+template <typename DT, int BITS, int NR, bool ROPE = false, bool SPLIT = false>   // NR: rows per thread (T <= NR * 256)
 __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* __restrict__ x, QuantGeom g, float clip,
                                                               uint16_t* __restrict__ scale,
                                                               uint16_t* __restrict__ zero,
@@ -461,37 +476,46 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
     // four 4-byte pieces of a packed row meet in one L2.  While a slice's rows are emitted, every
     // row's registers are refilled with the same row of the next slice: its loads are in flight
     // during the emit and its min / max pass starts without a wait.
-    const int nslice = static_cast<int>((static_cast<int64_t>(g.B) * g.H + 7) / 8) * 32;
+    const int plog = SPLIT ? g.parts_log2 : 0;
+    const int nslice = (static_cast<int>((static_cast<int64_t>(g.B) * g.H + 7) / 8) * 32) << plog;   // ids: slice * parts + part
     const int64_t nbh = static_cast<int64_t>(g.B) * g.H;
+    auto part_first = [&](int id) { return SPLIT ? (id & ((1 << plog) - 1)) * g.part_rows : 0; };        // first row of the id's part
+    auto part_len = [&](int id) { return SPLIT ? min(g.T - part_first(id), g.part_rows) : g.T; };       // rows of it
     // The slice's base is the same for the whole workgroup and a row's piece sits at a 32-bit byte
     // offset from it (the host checks T * row stride < 2^24 bytes): a load takes its address as
     // scalar base + vector offset, one 24-bit multiply-add per row.
-    auto slice_base = [&](int vb) -> const unsigned char* {   // slices past the last (batch, head) alias the last one
+    auto slice_base = [&](int id) -> const unsigned char* {   // slices past the last (batch, head) alias the last one
+        const int vb = id >> plog;
         const int quarter = (vb >> 3) & 3;
         const uint32_t bh = static_cast<uint32_t>(min(static_cast<int64_t>(vb >> 5) * 8 + (vb & 7), nbh - 1));
         const uint32_t b = g.dH.quot(bh), h = bh - b * g.dH.div;   // B * H < 2^31 on this path
-        return reinterpret_cast<const unsigned char*>(x + static_cast<int64_t>(b) * g.sb + static_cast<int64_t>(h) * g.sh + quarter * (ROPE ? 16 : 32));
+        return reinterpret_cast<const unsigned char*>(x + static_cast<int64_t>(b) * g.sb + static_cast<int64_t>(h) * g.sh +
+                                                      static_cast<int64_t>(part_first(id)) * g.st + quarter * (ROPE ? 16 : 32));
     };
     // first channel of the thread's piece, less the slice's own offset (quarter * 32, or quarter * 16 with ROPE)
     const int chan_t = ROPE ? (q4 >> 1) * 64 + (q4 & 1) * 8 : q4 * 8;
     const uint32_t st_bytes = static_cast<uint32_t>(g.st) * 2u, q_bytes = static_cast<uint32_t>(chan_t) * 2u;
-    auto row_offset = [&](int t) -> uint32_t {   // byte offset of the thread's piece of row min(t, T - 1)
-        return static_cast<uint32_t>(__umul24(static_cast<uint32_t>(min(t, g.T - 1)), st_bytes)) + q_bytes;
+    auto row_offset = [&](int t, int len) -> uint32_t {   // byte offset of the thread's piece of row min(t, len - 1) of a slice (part)
+        return static_cast<uint32_t>(__umul24(static_cast<uint32_t>(min(t, len - 1)), st_bytes)) + q_bytes;
     };
     typedef uint32_t U4 __attribute__((ext_vector_type(4)));
     U4 v[NR];
     {
         const unsigned char* base = slice_base(blockIdx.x);
+        const int len0 = part_len(blockIdx.x);
 #pragma unroll
         for (int i = 0; i < NR; ++i)   // rows past T re-read row T-1: min / max unchanged, never written
-            v[i] = *reinterpret_cast<const U4*>(base + row_offset(i * (kFThreads / 4) + row));
+            v[i] = *reinterpret_cast<const U4*>(base + row_offset(i * (kFThreads / 4) + row, len0));
     }
-    for (int vb = blockIdx.x; vb < nslice; vb += gridDim.x) {
+    for (int id = blockIdx.x; id < nslice; id += gridDim.x) {
+    const int vb = id >> plog;
     const int quarter = (vb >> 3) & 3;
     const int64_t bh = static_cast<int64_t>(vb >> 5) * 8 + (vb & 7);
     const bool live = bh < nbh;                         // a padding slice computes and writes nothing
-    const bool has_next = vb + static_cast<int>(gridDim.x) < nslice;
-    const unsigned char* next_base = slice_base(has_next ? vb + gridDim.x : vb);
+    const bool has_next = id + static_cast<int>(gridDim.x) < nslice;
+    const int next_id = has_next ? id + gridDim.x : id;
+    const unsigned char* next_base = slice_base(next_id);
+    const int t_first = part_first(id), t_len = part_len(id), next_len = part_len(next_id);
     int row_i = row;   // opaque per iteration: the row offsets below are recomputed, not kept in registers across the loop
     asm volatile("" : "+v"(row_i));
     if constexpr (ROPE) {
@@ -588,7 +612,7 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
                                   static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(wv)) * 1024u;
 #pragma unroll
             for (int i = 0; i < NP; ++i) {
-                const uint32_t off = row_offset(i * (kFThreads / 4) + row_i);
+                const uint32_t off = row_offset(i * (kFThreads / 4) + row_i, next_len);
                 const uint32_t ldsa = lds0 + static_cast<uint32_t>(i) * (kFThreads * 16);
                 if (i == 0)
                     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %2"
@@ -638,6 +662,37 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
         float z = fmaxf(fmaxf(z4.x, z4.y), fmaxf(z4.z, z4.w));
         a = row_reduce(a, OpMin(), INFINITY);
         z = row_reduce(z, OpMax(), -INFINITY);
+        if constexpr (SPLIT) {
+            if (p16 == 0 && live) {
+                // This part's extremes of channel c go out as two self-validating records; then the records of all
+                // parts of the slice are polled (device-scope loads, a bounded number of times) and folded.  The
+                // other parts are being worked on right now by other workgroups of this launch.
+                const unsigned long long tag = static_cast<unsigned long long>(g.epoch) << 32;
+                unsigned long long* mine = g.rec + (static_cast<int64_t>(id) * 32 + c) * 2;
+                __hip_atomic_store(mine, tag | __float_as_uint(a), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(mine + 1, tag | __float_as_uint(z), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const int nparts = 1 << plog;
+                const unsigned long long* first = g.rec + (static_cast<int64_t>(id & ~(nparts - 1)) * 32 + c) * 2;
+                bool ok = false;
+                float fa = a, fz = z;
+                for (int it = 0; it < g.spin_limit && !ok; ++it) {
+                    ok = true;
+                    fa = a; fz = z;
+                    for (int pp = 0; pp < nparts; ++pp) {
+                        const unsigned long long lo = __hip_atomic_load(first + pp * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        const unsigned long long hi = __hip_atomic_load(first + pp * 64 + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        ok = ok && static_cast<uint32_t>(lo >> 32) == g.epoch && static_cast<uint32_t>(hi >> 32) == g.epoch;
+                        // (a NaN extreme of any part stays one, as it does inside a part)
+                        const float pa = __uint_as_float(static_cast<uint32_t>(lo)), pz = __uint_as_float(static_cast<uint32_t>(hi));
+                        fa = (fa != fa || pa != pa) ? NAN : fminf(fa, pa);
+                        fz = (fz != fz || pz != pz) ? NAN : fmaxf(fz, pz);
+                    }
+                    if (!ok) __builtin_amdgcn_s_sleep(2);
+                }
+                if (ok) { a = fa; z = fz; }
+                else if (g.status) __hip_atomic_store(g.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);   // this call's result is not valid
+            }
+        }
         if (p16 == 0 && live) {
             const float x_min = rnd<DT>(a * clip);
             const float x_max = rnd<DT>(z * clip);
@@ -645,8 +700,10 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
             const float sc = rnd<DT>(diff * __fdiv_rn(1.0f, levels));
             const float zp = rnd<DT>(__fdiv_rn(-x_min, sc));
             const int64_t o = bh * g.D + (ROPE ? (c >> 4) * 64 + quarter * 16 + (c & 15) : quarter * 32 + c);
-            scale[o] = static_cast<uint16_t>(Cvt<DT>::from_float(sc));
-            zero[o] = static_cast<uint16_t>(Cvt<DT>::from_float(zp));
+            if (!SPLIT || t_first == 0) {   // (one of the parts writes them)
+                scale[o] = static_cast<uint16_t>(Cvt<DT>::from_float(sc));
+                zero[o] = static_cast<uint16_t>(Cvt<DT>::from_float(zp));
+            }
             s_s[c] = sc;
             s_z[c] = zp;
         }
@@ -715,7 +772,7 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
                 code[j] = ((f[j] >= th[0][j]) ? 1u : 0u) + ((f[j] >= th[1][j]) ? 1u : 0u) + ((f[j] >= th[2][j]) ? 1u : 0u);
         }
         // ROPE: the quad's bytes are two pairs, the lower-half pair at quarter * nb / 8 and the upper-half pair nb / 2 further
-        uint8_t* o = codes + (min(bh, nbh - 1) * g.T + min(t, g.T - 1)) * nb + (ROPE ? quarter * (nb / 8) : quarter * (nb / 4));
+        uint8_t* o = codes + (min(bh, nbh - 1) * g.T + t_first + min(t, t_len - 1)) * nb + (ROPE ? quarter * (nb / 8) : quarter * (nb / 4));
         if constexpr (BITS == 1) {
             // The byte is built by eight add-with-carry steps, w = w + w + (f[j] >= th[j]): each
             // comparison leaves its lane mask in a scalar register pair of its own and the add
@@ -752,10 +809,10 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
             w |= static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(w), 0xB1, 0xf, 0xf, true));
             w |= static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(w), 0x4E, 0xf, 0xf, true));
             if constexpr (ROPE) {
-                if ((q4 & 1) == 0 && t < g.T && live)
+                if ((q4 & 1) == 0 && t < t_len && live)
                     *reinterpret_cast<uint16_t*>(o + (q4 >> 1) * (nb / 2)) = static_cast<uint16_t>(w >> (8 * q4));
             } else {
-                if (q4 == 0 && t < g.T && live) *reinterpret_cast<uint32_t*>(o) = w;
+                if (q4 == 0 && t < t_len && live) *reinterpret_cast<uint32_t*>(o) = w;
             }
         } else {
             const uint32_t b0 = (code[0] << 6) | (code[1] << 4) | (code[2] << 2) | code[3];
@@ -763,15 +820,15 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
             const uint32_t half = b0 | (b1 << 8);
             const uint32_t other = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(half), 0xB1, 0xf, 0xf, true));
             if constexpr (ROPE) {
-                if ((q4 & 1) == 0 && t < g.T && live) *reinterpret_cast<uint32_t*>(o + (q4 >> 1) * (nb / 2)) = half | (other << 16);
+                if ((q4 & 1) == 0 && t < t_len && live) *reinterpret_cast<uint32_t*>(o + (q4 >> 1) * (nb / 2)) = half | (other << 16);
             } else {
-                if ((q4 & 1) == 0 && t < g.T && live) reinterpret_cast<uint32_t*>(o)[q4 >> 1] = half | (other << 16);
+                if ((q4 & 1) == 0 && t < t_len && live) reinterpret_cast<uint32_t*>(o)[q4 >> 1] = half | (other << 16);
             }
         }
         // the row is packed: its registers take the same row of the next slice
         if (has_next) {
             if (i < NP) v[i] = *reinterpret_cast<const U4*>(stage + (i * kFThreads + tid) * 16);
-            else v[i] = *reinterpret_cast<const U4*>(next_base + row_offset(t));
+            else v[i] = *reinterpret_cast<const U4*>(next_base + row_offset(t, next_len));
         }
     }
     }
@@ -797,11 +854,11 @@ static int allow_dynamic_lds(const void* kernel, int bytes) {
     return CQ_OK;
 }
 
-template <typename DT, int BITS, int NR, bool ROPE>
+template <typename DT, int BITS, int NR, bool ROPE, bool SPLIT = false>
 static int launch_fused(dim3 grid, hipStream_t st, const uint16_t* xp, const QuantGeom& g, float clip, uint16_t* sp,
                         uint16_t* zp, uint8_t* codes, const RopeArgs& ra) {
     constexpr int lds = fused_stage_rows(NR, ROPE) * kFThreads * 16;
-    auto kf = fused_pack_kernel<DT, BITS, NR, ROPE>;
+    auto kf = fused_pack_kernel<DT, BITS, NR, ROPE, SPLIT>;
     if (lds) {
         const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kf), lds);
         if (rc != CQ_OK) return rc;
@@ -824,6 +881,68 @@ static int persistent_units() {
     }
     cached.store(cu, std::memory_order_relaxed);
     return cu;
+}
+
+// ---- a token axis longer than one workgroup's registers: several workgroups per slice (SPLIT) ----------------
+// Parts per slice (a power of two up to 32, so that it divides the persistent grid), rows per part and per thread:
+// the choice that loads the fewest rows (a thread's rows past its part's end repeat the part's last row).  Only with
+// more than eight rows per thread, the instantiations that stage the next slice's rows through LDS: measured against
+// the three launches (partial min / max, statistics, emit - whose second read of x comes from the memory-side cache)
+// on one device, 1 bit, (batch, tokens, 8 heads): strided view of a fused projection (16, 9 984) 105 against 126 us,
+// (64, 5 000) 224 against 263 us, contiguous (16, 9 984) 123 against 123 us; with eight rows per thread and no
+// staging (8, 32 768) 265 against 205 us.
+struct SplitPlan { int plog, part_rows, nr; };
+static bool split_plan(int T, SplitPlan* sp) {
+    static const int kRowOptions[2] = {10, 13};
+    int64_t best = -1;
+    for (int plog = 1; plog <= 5; ++plog) {
+        const int parts = 1 << plog;
+        const int rows = (T + parts - 1) / parts;
+        if (rows > kFMaxT || static_cast<int64_t>(parts - 1) * rows >= T) continue;
+        const int need = (rows + kFThreads / 4 - 1) / (kFThreads / 4);
+        int nr = 0;
+        for (int o : kRowOptions) if (!nr && o >= need) nr = o;
+        if (need <= 8) continue;   // (would be the unstaged instantiation)
+        const int64_t cost = static_cast<int64_t>(nr) * parts;
+        if (best < 0 || cost < best) { best = cost; sp->plog = plog; sp->part_rows = rows; sp->nr = nr; }
+    }
+    return best >= 0;
+}
+static size_t split_records_bytes(int B, int H, int plog) {
+    return ((static_cast<size_t>(B) * H + 7) / 8 * 32 << plog) * 32 * 2 * sizeof(unsigned long long);
+}
+
+// The wait of a part for the others is bounded; a lane that gives up sets a word of pinned host memory (one per
+// device, allocated at the first such call outside a stream capture, never freed).  The next call on the device
+// finds it, reports CQ_ERR_LAUNCH once, and the process goes on with the three-launch path.
+constexpr int kQMaxDevices = 64;
+static std::atomic<int*> g_qstatus[kQMaxDevices];
+static std::atomic<bool> g_split_off{false};
+static std::atomic<uint32_t> g_qepoch{0x51ab0000u};
+static std::atomic<int> g_qspin{1 << 18};
+
+static int* split_status_word(hipStream_t st) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kQMaxDevices) return nullptr;
+    int* p = g_qstatus[dev].load(std::memory_order_acquire);
+    if (p) return p;
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;   // not while the stream is being recorded
+    if (hipStreamIsCapturing(st, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    void* raw = nullptr;
+    if (hipHostMalloc(&raw, 64, hipHostMallocDefault) != hipSuccess || !raw) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    *static_cast<volatile int*>(raw) = 0;
+    int* expected = nullptr;
+    if (!g_qstatus[dev].compare_exchange_strong(expected, static_cast<int*>(raw), std::memory_order_acq_rel)) {
+        (void)hipHostFree(raw);   // another host thread was first
+        return expected;
+    }
+    return static_cast<int*>(raw);
 }
 
 static bool one_pass_shape(const QuantGeom& g, const uint8_t* codes) {
@@ -866,6 +985,44 @@ static int run_quant(const void* x, QuantGeom g, int bits, float clip, uint8_t* 
 #undef CQ_FUSED
         CQ_LAUNCH_CHECK();
         return CQ_OK;
+    }
+    SplitPlan spl;
+    if (!xq && !rope && g.D == 128 && g.T > kFMaxT && split_plan(g.T, &spl) && !g_split_off.load(std::memory_order_relaxed) &&
+        (reinterpret_cast<uintptr_t>(codes) & 3u) == 0 && static_cast<int64_t>(g.B) * g.H < (static_cast<int64_t>(1) << 26) &&
+        g.st > 0 && g.st * 2 < (1 << 24) && static_cast<int64_t>(spl.part_rows) * g.st * 2 < (static_cast<int64_t>(1) << 31)) {
+        // Still one pass over x: the slices are split along the token axis between workgroups of one persistent
+        // launch, which exchange their channel min / max inside it.
+        int* status = split_status_word(st);
+        if (status) {
+            if (*static_cast<volatile int*>(status) != 0) {
+                *static_cast<volatile int*>(status) = 0;
+                g_split_off.store(true, std::memory_order_relaxed);
+                return CQ_ERR_LAUNCH;   // an earlier split pass did not complete: its output is not valid
+            }
+            const int64_t nids = ((static_cast<int64_t>(g.B) * g.H + 7) / 8 * 32) << spl.plog;
+            const int cu = persistent_units();
+            const int64_t fmax = cu >= 32 ? cu / 32 * 32 : 32;
+            const dim3 fgrid(static_cast<unsigned>(nids < fmax ? nids : fmax));
+            g.parts_log2 = spl.plog;
+            g.part_rows = spl.part_rows;
+            g.rec = reinterpret_cast<unsigned long long*>(ws);
+            uint32_t ep = g_qepoch.fetch_add(1, std::memory_order_relaxed) + 1;
+            g.epoch = ep ? ep : g_qepoch.fetch_add(1, std::memory_order_relaxed) + 1;
+            g.spin_limit = g_qspin.load(std::memory_order_relaxed);
+            g.status = status;
+            const RopeArgs ra{};
+            int rc = CQ_OK;
+#define CQ_SPLIT(B_, N_) rc = launch_fused<DT, B_, N_, false, true>(fgrid, st, xp, g, clip, sp, zp, codes, ra)
+            if (bits == 1) {
+                if (spl.nr == 10) CQ_SPLIT(1, 10); else CQ_SPLIT(1, 13);
+            } else {
+                if (spl.nr == 10) CQ_SPLIT(2, 10); else CQ_SPLIT(2, 13);
+            }
+#undef CQ_SPLIT
+            if (rc != CQ_OK) return rc;
+            CQ_LAUNCH_CHECK();
+            return CQ_OK;
+        }
     }
     hipLaunchKernelGGL(minmax_partial_kernel<DT>, grid, dim3(kQThreads), 0, st, xp, g, ws);
     CQ_LAUNCH_CHECK();
@@ -1140,7 +1297,23 @@ size_t cq_quantize_pack_workspace(int B, int T, int H, int D) {
     if (B < 1 || T < 1 || H < 1 || D < 1) return 0;
     // partial min / max per chunk, then three thresholds per channel (+ one row of statistics in the
     // storage dtype for the whole-tensor mode of cq_quant_tensor)
-    return (static_cast<size_t>(B) * H * (static_cast<size_t>(cq::pick_chunks(B, T, H)) * 2 + 3) + 4) * D * sizeof(float);
+    size_t need = (static_cast<size_t>(B) * H * (static_cast<size_t>(cq::pick_chunks(B, T, H)) * 2 + 3) + 4) * D * sizeof(float);
+    // (the records that the parts of a split slice exchange, when the one-pass kernel takes a long token axis)
+    cq::SplitPlan spl;
+    if (D == 128 && T > cq::kFMaxT && cq::split_plan(T, &spl)) {
+        const size_t rec = cq::split_records_bytes(B, H, spl.plog);
+        if (rec > need) need = rec;
+    }
+    return need;
+}
+
+int cq_quantize_pack_wait_polls(int polls) {
+    const int before = cq::g_qspin.load(std::memory_order_relaxed);
+    if (polls >= 0) {
+        cq::g_qspin.store(polls, std::memory_order_relaxed);
+        cq::g_split_off.store(false, std::memory_order_relaxed);
+    }
+    return before;
 }
 
 int cq_quantize_pack(const void* x, int dtype, int B, int T, int H, int D, int64_t stride_b, int64_t stride_t,

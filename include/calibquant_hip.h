@@ -67,6 +67,18 @@ int cq_quantize_pack(const void* x, int dtype, int B, int T, int H, int D,
                      uint8_t* codes, void* scale, void* zero,
                      void* workspace, size_t workspace_bytes, cq_stream_t stream);
 
+/* With D = 128 and more than 3 328 tokens (what one workgroup's registers hold of a slice of 32 channels),
+ * cq_quantize_pack still reads x once: two to thirty-two workgroups of its persistent launch share a slice along
+ * the token axis and exchange the channels' minima and maxima through the workspace inside the launch.  The wait
+ * for the other parts is bounded: after `polls` polls (about a microsecond each; default 262 144) a workgroup goes
+ * on with what it has and sets a word of pinned host memory (64 bytes per device, allocated at the first such
+ * call outside a stream capture and kept until the process ends).  The next such call on that device then returns
+ * CQ_ERR_LAUNCH once (the previous call's output is not valid) and the process goes on with three launches per
+ * tensor (partial min / max, statistics, emit; x read twice).  This call sets the bound (polls >= 0; it also
+ * re-enables the single launch after a give-up) and returns the previous one; polls < 0 only queries.  No
+ * counterpart in the reference, whose quant() is a chain of whole-tensor torch ops (calibquant.py:24-42). */
+int cq_quantize_pack_wait_polls(int polls);
+
 /* ------------------------------------------------------------------------
  * Prefill, keys: rotary embedding fused into the quantise-and-pack pass.
  * Replaces, for the image slice of the key tensor, the rotary embedding of

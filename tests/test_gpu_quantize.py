@@ -144,3 +144,72 @@ def test_quantize_pack_full_size_properties(ops, bits):
     codes2, _, _ = ops.quantize_pack(deq.transpose(1, 2), bits, 1.0)
     un2 = ((codes2[..., None] >> shifts) & L).reshape(B, H, T, D)
     assert (un2 != un).float().mean().item() < 2e-3
+
+
+# Token axes beyond what one workgroup's registers hold of a slice (3 328 rows): the one-pass kernel splits a slice
+# between 2, 4, ... workgroups of its launch when a part then has more than 2 048 rows (parts x rows per part ->
+# rows per thread); the other shapes take three launches.
+LONG_SHAPES = [(2, 9984, 8, 128),    # 4 x 2496 -> 10: the 26B prompt's token count
+               (3, 3329, 2, 128),    # just beyond one workgroup: three launches
+               (1, 13000, 1, 128),   # 4 x 3250 -> 13
+               (1, 40000, 1, 128),   # 16 x 2500 -> 10
+               (9, 5000, 8, 128),    # 2 x 2500 -> 10; 288 slices x 2 parts: more ids than workgroups, 3 steps
+               (2, 7000, 8, 128)]    # three launches
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("bits", [1, 2])
+@pytest.mark.parametrize("shape", LONG_SHAPES)
+def test_quantize_pack_long_token_axis_bit_exact(ops, shape, bits, dtype):
+    B, T, H, D = shape
+    print(f"case quantize_pack long shape={shape} bits={bits} dtype={dtype}", flush=True)
+    k, _ = O.synth_kv(B, T, H, D, dtype, seed=T + bits)
+    clip = CLIPS[bits][0]
+    codes, s, z = ops.quantize_pack(to_gpu(k, dtype), bits, clip)
+    torch.cuda.synchronize()
+    oc, os_, oz = O.quantize_pack(k, bits, clip, dtype)
+    assert same_bits(to_np(s), os_) and same_bits(to_np(z), oz)
+    assert np.array_equal(codes.cpu().numpy(), oc)
+
+
+def test_quantize_pack_long_token_axis_strided_view(ops):
+    B, N, Hkv, G, D, S, T = 2, 10100, 2, 4, 128, 41, 9984
+    rng = np.random.default_rng(5)
+    qkv = O.round_to(rng.standard_normal((B, N, Hkv, G + 2, D), dtype=np.float32), "bf16")
+    t = to_gpu(qkv, "bf16")
+    view = t[:, S:S + T, :, G, :]
+    assert not view.is_contiguous()
+    codes, s, z = ops.quantize_pack(view, 1, 0.5)
+    oc, os_, oz = O.quantize_pack(qkv[:, S:S + T, :, G], 1, 0.5, "bf16")
+    assert same_bits(to_np(s), os_) and same_bits(to_np(z), oz)
+    assert np.array_equal(codes.cpu().numpy(), oc)
+
+
+def test_quantize_pack_split_slices_give_up_and_the_host_reports_it(ops):
+    """The parts of a split slice wait for each other a bounded number of polls.  With the bound at zero every
+    part goes on alone (the kernel ends normally; its statistics are those of single parts, i.e. not valid): the
+    call returns success, the next call on the device reports the failure once, and from then on long token axes
+    take the three-launch path - bit-exact - until the bound is set again."""
+    from calibquant_amd import _lib
+    lib = _lib.load()
+    B, T, H, D = 2, 9984, 2, 128
+    k, _ = O.synth_kv(B, T, H, D, "bf16", seed=31)
+    x = to_gpu(k, "bf16")
+    oc, os_, oz = O.quantize_pack(k, 1, 0.5, "bf16")
+
+    def check():
+        codes, s, z = ops.quantize_pack(x, 1, 0.5)
+        torch.cuda.synchronize()
+        assert same_bits(to_np(s), os_) and same_bits(to_np(z), oz)
+        assert np.array_equal(codes.cpu().numpy(), oc)
+    check()
+    before = lib.cq_quantize_pack_wait_polls(0)
+    try:
+        ops.quantize_pack(x, 1, 0.5)          # launched; every part gives up
+        torch.cuda.synchronize()
+        with pytest.raises(_lib.CalibQuantError):
+            ops.quantize_pack(x, 1, 0.5)      # the host finds the word set
+        check()                               # three launches from here on
+    finally:
+        lib.cq_quantize_pack_wait_polls(before)
+    check()
