@@ -479,12 +479,15 @@ __global__ __launch_bounds__(kFThreads) void fused_pack_kernel(const uint16_t* _
     // during the emit and its min / max pass starts without a wait.
     const int plog = SPLIT ? g.parts_log2 : 0;
     const int64_t nbh = static_cast<int64_t>(g.B) * g.H;
-    // Slice vb -> (quarter, (batch, head) pair).  Workgroup l of the launch runs on die l % 8, and a workgroup's
-    // slices are a multiple of 8 apart, so the low three bits of vb are the die.  The four quarters of a pair always
-    // share a die (their 4-byte pieces of a packed row meet in one L2, and two quarters share every 128-byte line
-    // of x).  Narrow map: consecutive pairs on consecutive dies.  Wide map: eight consecutive pairs - with eight
-    // heads, a whole batch row - on one die, whose 32 workgroups then read one contiguous span of a (B, T, H, D)
-    // tensor together instead of every die reading a 256-byte piece out of every 2 KB.
+    // Slice vb -> (quarter, (batch, head) pair).  Workgroup l of the launch runs on die l % 8 and its ids are a
+    // multiple of 8 apart, so the low three bits of an id are the die: of an unsplit slice the low three bits of vb,
+    // of a slice split four ways the part and the lowest bit of vb.  The four quarters of a pair always share a
+    // die (their 4-byte pieces of a packed row meet in one L2, and two quarters share every 128-byte line of x).
+    // Narrow map: the low bits of vb are the low bits of the pair index - with eight heads, of the head.  Wide
+    // map: they select among eight runs of eight consecutive pairs - with eight heads, among batch rows - and the
+    // place in the run comes from bits 5-7.  For split slices of a contiguous (B, T, H, D) tensor the wide map
+    // puts all heads of a token row (one contiguous 2 KB) on one die, where the narrow one spreads them over two
+    // or more; the host picks it there (measured, see wide_map_for()).
     const int wide = g.wide_map;
     const int nslice = (wide ? static_cast<int>((nbh + 63) / 64) * 256 : static_cast<int>((nbh + 7) / 8) * 32) << plog;   // ids: slice * parts + part
     auto slice_of = [&](int vb, int& quarter) -> int64_t {
