@@ -221,7 +221,7 @@ def prefill_leg(torch, ops, shape, bits, steps=40, warmup=10, contiguous=False, 
         inv = 1.0 / (1e6 ** (torch.arange(0, D, 2, device=dev).float() / D))
         emb = torch.cat([torch.outer(t, inv)] * 2, dim=-1)
         cos, sin = emb.cos().to(torch.bfloat16), emb.sin().to(torch.bfloat16)
-        k_rot = torch.empty((B, T, Hkv, D), device=dev, dtype=torch.bfloat16)
+        k_rot = ops.empty_token_rows(B, T, Hkv, D, torch.bfloat16, dev)   # as the patched forward allocates it
         ms_f = _time_fn(torch, lambda: ops.rope_quantize_pack(k_view, cos, sin, 41, k_rot, bits, clip), steps, warmup)
         ms_r = _time_fn(torch, lambda: ops.rope_rows(k_view, cos, sin, 41, out=k_rot), steps, warmup)
         ms_q = _time_fn(torch, lambda: ops.quantize_pack(k_rot, bits, clip), steps, warmup)

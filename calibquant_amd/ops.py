@@ -38,6 +38,16 @@ def _workspace(nbytes: int, device) -> Optional[torch.Tensor]:
     return torch.empty(nbytes, dtype=torch.uint8, device=device)
 
 
+def empty_token_rows(B: int, T: int, H: int, D: int, dtype, device) -> torch.Tensor:
+    """An uninitialised (B, T, H, D) tensor for keys or values that the quantiser will read: token rows of
+    H * D elements, plus 128 bytes of padding per row where rows would otherwise lie a multiple of 2 KB apart -
+    the one-pass quantiser's slices then meet too few memory channels (measured at batch 64 x 3 328 tokens x 8
+    heads: 129 us per tensor contiguous, 105 us padded).  The result is a view; D stays contiguous."""
+    row = H * D
+    pad = 64 if (row * torch.empty((), dtype=dtype).element_size()) % 2048 == 0 else 0
+    return torch.empty((B, T, row + pad), dtype=dtype, device=device)[:, :, :row].unflatten(2, (H, D))
+
+
 def quantize_pack(x: torch.Tensor, bits: int, clip: float) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """Per-channel min-max quantise and bit-pack one K or V tensor.
 

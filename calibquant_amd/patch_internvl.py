@@ -202,12 +202,7 @@ def forward_internlm2_calibquant(self, hidden_states: torch.Tensor, attention_ma
         ops.rope_rows_grouped(qkv[..., :G, :], cos, sin, position_ids, out=q_rot)   # all query heads: one launch
         query_states = q_rot.view(bsz, q_len, Hq, D).transpose(1, 2)               # (B, Hq, q, D)
         k_raw = qkv[..., -2, :]                                                    # (B, q, Hkv, D), un-rotated
-        # (rotated keys: a token row of Hkv * D elements, plus 128 bytes where rows would otherwise be a multiple of
-        # 2 KB apart - the quantiser's slices then meet too few memory channels: 129 against 105 us per tensor at
-        # batch 64 x 3 328 tokens x 8 heads)
-        row = Hkv * D
-        pad = 64 if (row * qkv.element_size()) % 2048 == 0 else 0
-        k_rot = torch.empty((bsz, q_len, row + pad), dtype=qkv.dtype, device=qkv.device)[:, :, :row].unflatten(2, (Hkv, D))
+        k_rot = ops.empty_token_rows(bsz, q_len, Hkv, D, qkv.dtype, qkv.device)    # (padded rows where that helps the quantiser)
         key_states = k_rot.transpose(1, 2)                                         # filled in the prefill branch
     else:
         query_states = qkv[..., :G, :].reshape(bsz, q_len, Hq, D).transpose(1, 2)  # (B, Hq, q, D)
