@@ -29,8 +29,9 @@ void check(int rc, const char* what) {
 class LayerStep {
   public:
     // `decode_args_addr`, `decode_args_bytes`: address and size of a filled `cq_decode_args` (the prepared call of the Python
-    // path, no workspace, no mask, no device row count); it is copied.  The caller keeps the
-    // tensors it points at (packed codes, statistics) alive for the life of this object.
+    // path, no mask, no device row count; a chunked call brings its workspace, whose size depends on the packed
+    // tokens only); it is copied.  The caller keeps the tensors it points at (packed codes, statistics,
+    // workspace) alive for the life of this object.
     // cos, sin: rotary tables (rows, D) in the storage dtype.  k_win, v_win: the window buffers
     // (B, Hkv, capacity, D) whose first `len` rows are filled.  ramp: int64 device vector whose
     // cell i holds i (the row index is read on the device).
@@ -41,8 +42,8 @@ class LayerStep {
         TORCH_CHECK(decode_args_bytes == sizeof(a_), "LayerStep: argument block of ", decode_args_bytes,
                     " bytes, the library's is ", sizeof(a_));
         std::memcpy(&a_, reinterpret_cast<const void*>(decode_args_addr), sizeof(a_));
-        TORCH_CHECK(a_.workspace_bytes == 0 && a_.mask == nullptr && a_.r_dev == nullptr,
-                    "LayerStep: the prepared call must need no workspace, mask or device row count");
+        TORCH_CHECK(a_.mask == nullptr && a_.r_dev == nullptr && (a_.workspace_bytes == 0 || a_.workspace != nullptr),
+                    "LayerStep: the prepared call must need no mask or device row count");
         dtype_ = a_.dtype == CQ_BF16 ? at::kBFloat16 : at::kHalf;
         TORCH_CHECK(k_.is_cuda() && k_.dim() == 4 && k_.sizes() == v_.sizes() && k_.strides() == v_.strides() &&
                         k_.stride(3) == 1 && k_.size(0) == a_.B && k_.size(1) == a_.Hkv && k_.size(3) == a_.D &&

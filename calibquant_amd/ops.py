@@ -48,6 +48,25 @@ def empty_token_rows(B: int, T: int, H: int, D: int, dtype, device) -> torch.Ten
     return torch.empty((B, T, row + pad), dtype=dtype, device=device)[:, :, :row].unflatten(2, (H, D))
 
 
+_decode_ws = {}
+
+
+def _decode_workspace(nbytes: int, device) -> Optional[torch.Tensor]:
+    """The workspace of a chunked decode call: one buffer per (device, stream), shared by every call made on
+    that stream (the layers of a model run one after the other; calls on one stream are ordered) and grown when
+    a call needs more.  A call keeps a reference to the buffer it was prepared with, so a buffer that has been
+    outgrown lives as long as the calls that use it.  Nothing in it has to survive from one call to the next."""
+    if nbytes == 0:
+        return None
+    dev = torch.device(device)
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(dev).cuda_stream)
+    ws = _decode_ws.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        _decode_ws[key] = ws
+    return ws
+
+
 def quantize_pack(x: torch.Tensor, bits: int, clip: float) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """Per-channel min-max quantise and bit-pack one K or V tensor.
 
@@ -349,12 +368,13 @@ class DecodeCall:
         # static_scratch: `cq_decode_attn_static`, whose scratch is a static device buffer inside the
         # library - no workspace tensor, nothing allocated per call; calls on one GPU must not overlap
         self._entry = self._lib.cq_decode_attn_static if static_scratch else self._lib.cq_decode_attn
-        ws = None if static_scratch else _workspace(self._lib.cq_decode_attn_workspace(C.byref(a)), q.device)
+        need = 0 if static_scratch else self._lib.cq_decode_attn_workspace(C.byref(a))
+        ws = _decode_workspace(need, q.device)
         if ws is not None:
-            a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+            a.workspace, a.workspace_bytes = ws.data_ptr(), need
             keep.append(ws)
         self.args, self._ref, self._keep, self.out, self.device = a, C.byref(a), keep, out, q.device
-        self.workspace, self.workspace_bytes = ws, 0 if ws is None else ws.numel()
+        self.workspace, self.workspace_bytes = (None if ws is None else ws[:need]), need
 
     def plan(self) -> dict:
         """What the launch will be for the prepared arguments (`cq_decode_attn_plan`): threads per

@@ -301,12 +301,13 @@ def forward_internlm2_calibquant(self, hidden_states: torch.Tensor, attention_ma
 def _attend(self, q1, k_res, v_res, mask):
     """The fused decode attention of one step over the module's packed state and the full-precision
     window (k_res, v_res): q1 (B, Hq, D) -> (B, Hq, D).  In the steady state (no mask, same batch and
-    dtype, no workspace) the prepared call of the previous step is re-aimed at this step's tensors."""
+    dtype) the prepared call of the previous step is re-aimed at this step's tensors (a chunked call keeps
+    its plan and its workspace: both depend on the packed tokens only, once the window has a row)."""
     bsz = q1.shape[0]
     S, T = self.sprompt_len, self.image_token_num
     R = k_res.shape[2]
     call = getattr(self, "_cq_call", None)
-    if (mask is None and call is not None and call.args.B == bsz and call.workspace_bytes == 0
+    if (mask is None and call is not None and call.args.B == bsz and call.args.R > 0
             and q1.is_contiguous() and call.args.dtype == (0 if q1.dtype == torch.bfloat16 else 1)):
         return call.step(q1, k_res, v_res, torch.empty_like(q1))
     stats = self._cq_stats if T > 0 else (None,) * 4
@@ -364,7 +365,7 @@ def _decode_step_fused(self, qkv, position_ids, past_key_value, attention_mask, 
         mask = attention_mask[:, 0, 0, :]
     out = _attend(self, q1, k_res, v_res, mask)
     call = getattr(self, "_cq_call", None)
-    if (mask is None and use_cache and call is not None and call.workspace_bytes == 0 and call.args.B == bsz
+    if (mask is None and use_cache and call is not None and call.args.B == bsz
             and not getattr(self, "cq_no_step_shim", False)):
         # from the next token on the host shim runs this whole function in one call; it takes over the
         # window buffers (this step's past_key_value are views of them) and keeps `call`'s tensors alive

@@ -166,6 +166,46 @@ def test_fused_decode_step_equals_the_unfused_op_chain(dtype):
         assert torch.equal(outs[0], outs[other])
 
 
+def test_fused_decode_step_on_a_chunked_context():
+    """A context whose packed tokens take several chunks (a call with a workspace): the steady-state decode step
+    goes through the host shim and the re-aimed call object all the same, and both give the bits of the path that
+    prepares a new call on every step."""
+    from calibquant_amd import patch_internvl as pi
+    from calibquant_amd.internlm2 import InternLM2Attention, InternLM2Config
+    cfg = InternLM2Config.tiny()
+    dtype = torch.bfloat16
+    B, S, T, TXT = 2, 4, 20000, 9
+    N = S + T + TXT
+    outs = []
+    for mode in ("shim", "call", "fresh"):
+        torch.manual_seed(11)
+        att = InternLM2Attention(cfg).cuda().to(dtype)
+        att.cq_sprompt_len, att.cq_image_token_num = S, T
+        att.cq_no_step_shim = mode != "shim"
+        x = torch.randn(B, N, cfg.hidden_size, device="cuda", dtype=dtype)
+        pos = torch.arange(N, device="cuda")[None].expand(B, N)
+        with torch.no_grad():
+            _, _, past = pi.forward_internlm2_calibquant(att, x, None, pos, None, False, True)
+            step_out = []
+            for i in range(12):
+                xd = torch.randn(B, 1, cfg.hidden_size, device="cuda", dtype=dtype)
+                posd = torch.full((B, 1), N + i, device="cuda", dtype=torch.long)
+                if mode == "fresh":
+                    att._cq_call = None     # a new prepared call (and plan) on every step
+                o, _, past = pi.forward_internlm2_calibquant(att, xd, None, posd, past, False, True)
+                step_out.append(o.clone())
+                if i == 0:
+                    plan = att._cq_call.plan()
+                    assert plan["chunks"] > 1 and att._cq_call.workspace_bytes > 0
+        if mode == "shim":
+            assert att._cq_step[0].steps == 11
+        else:
+            assert "_cq_step" not in att.__dict__
+        outs.append(torch.stack(step_out))
+    assert torch.isfinite(outs[0].float()).all()
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+
+
 def test_patched_model_without_image_tokens_equals_the_fp_model():
     """With zero packed tokens the quantised path is plain attention over the fp window."""
     from calibquant_amd import patch_internvl as pi
