@@ -1016,7 +1016,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                     // those of chunk s, a bounded number of times (workgroups that are not all resident together -
                     // a smaller device than planned for - must not spin for ever; giving up ends this workgroup
                     // without a result and tells the host), folds them and leaves the unit's min / max in LDS.
-                    float* fold = red + 4 * HPB;           // 2 * HPB floats, then the verdict
+                    float* fold = red + 4 * HPB;           // 2 * HPB floats, then whether the wait succeeded
                     int* flag = reinterpret_cast<int*>(fold + 2 * HPB);
                     if (wv == 0) {
                         const unsigned long long* pr = g.rec + ((unit * HPB) * g.nsplit + min(lane, g.nsplit - 1)) * 2;
