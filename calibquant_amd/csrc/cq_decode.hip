@@ -1238,11 +1238,20 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                 }
                 // One pass over the TPW tokens of unit u: the sum of the entries each of the lane's bit lanes picks,
                 // as packed fp16 (GPW entries of at most 4 terms each, added pairwise).
-                auto v_pass = [&](int u, f16x2_t (&sum)[L::MPL][L::HW]) {
+                struct PreV { HWv e[4]; WG cw; };
+                auto load_pre = [&](int u, PreV& p) {
+                    const int tl = u * L::TPW;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) p.e[i] = *reinterpret_cast<const HWv*>(slot(vs0 + tl + 4 * bg + i));
+                    p.cw = *reinterpret_cast<const WG*>(vst + (u * NB + j) * L::TPW);
+                };
+                // A pass in three steps, so that two passes can be woven together: the table of the second is built and
+                // written while the look-ups of the first are in flight (the LDS executes a wave's instructions in
+                // order: the second table's write lands after the first pass's reads).
+                auto v_build = [&](int u, const PreV& pre) {
                     const int tl = u * L::TPW;        // token offset inside the block
+                    (void)tl;
                     if (bg < L::GPW) {
-                        // entry `be` of group `bg`: fp16 sum of the e values its bits select
-                        // (VTOK: of e times the token's scale for the channel group, per group)
                         f16x2_t val[L::NGRP][L::HW];
 #pragma unroll
                         for (int gi = 0; gi < L::NGRP; ++gi)
@@ -1251,7 +1260,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
                             const unsigned char* sl = slot(vs0 + tl + 4 * bg + i);
-                            const HWv e = *reinterpret_cast<const HWv*>(sl);
+                            const HWv e = VTOK ? *reinterpret_cast<const HWv*>(sl) : pre.e[i];
                             if constexpr (VTOK) {
                                 const uint2 sc = *reinterpret_cast<const uint2*>(sl + 8);
                                 const f16x2_t s01 = __builtin_bit_cast(f16x2_t, sc.x), s23 = __builtin_bit_cast(f16x2_t, sc.y);
@@ -1275,14 +1284,11 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                             reinterpret_cast<HWv*>(wtab)[(gi * L::GPW + bg) * 16 + be] = o;
                         }
                     }
-                    const WG cw = *reinterpret_cast<const WG*>(vst + (u * NB + j) * L::TPW);
                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                     __builtin_amdgcn_wave_barrier();
                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-                    // The GPW entries a bit lane picks in this pass (each at most 4) are first
-                    // added as packed fp16 pairs, pairwise; one mixed-precision FMA per head then
-                    // moves the sum into the fp32 accumulator.
-                    f16x2_t pk[L::MPL][L::GPW][L::HW];
+                };
+                auto v_lookups = [&](const WG& cw, f16x2_t (&pk)[L::MPL][L::GPW][L::HW]) {
 #pragma unroll
                     for (int gq = 0; gq < L::GPW; ++gq) {
                         const uint32_t tbase = wtab_addr + static_cast<uint32_t>((cgrp * L::GPW + gq) * 16 * L::ESZH);
@@ -1296,6 +1302,8 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                             for (int k = 0; k < L::HW; ++k) pk[m][gq][k] = __builtin_bit_cast(f16x2_t, e.w[k]);
                         }
                     }
+                };
+                auto v_reduce = [&](f16x2_t (&pk)[L::MPL][L::GPW][L::HW], f16x2_t (&sum)[L::MPL][L::HW]) {
 #pragma unroll
                     for (int m = 0; m < L::MPL; ++m) {
 #pragma unroll
@@ -1307,6 +1315,13 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
 #pragma unroll
                         for (int k = 0; k < L::HW; ++k) sum[m][k] = pk[m][0][k];
                     }
+                };
+                auto v_pass = [&](int u, f16x2_t (&sum)[L::MPL][L::HW], const PreV& pre, auto&& after_lookups) {
+                    f16x2_t pk[L::MPL][L::GPW][L::HW];
+                    v_build(u, pre);
+                    v_lookups(pre.cw, pk);
+                    after_lookups();
+                    v_reduce(pk, sum);
                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                     __builtin_amdgcn_wave_barrier();
                 };
@@ -1322,12 +1337,24 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                         }
                 };
                 int u = wvu;   // wave-uniform loop control
+                // the slot entries and code words of a pass are read while the pass before it waits for its look-ups
+                PreV cur, nxt;
+                if (u * L::TPW < vn) load_pre(u, cur);
                 {
                     // two passes per fp32 accumulation: the sums of 2 * TPW tokens meet as packed fp16 first
                     for (; (u + kNW) * L::TPW < vn; u += 2 * kNW) {
                         f16x2_t s0[L::MPL][L::HW], s1[L::MPL][L::HW];
-                        v_pass(u, s0);
-                        v_pass(u + kNW, s1);
+                        f16x2_t pk0[L::MPL][L::GPW][L::HW], pk1[L::MPL][L::GPW][L::HW];
+                        v_build(u, cur);
+                        v_lookups(cur.cw, pk0);
+                        load_pre(u + kNW, nxt);
+                        v_build(u + kNW, nxt);           // (its table write queues behind the look-ups above)
+                        v_lookups(nxt.cw, pk1);
+                        if ((u + 2 * kNW) * L::TPW < vn) load_pre(u + 2 * kNW, cur);
+                        v_reduce(pk0, s0);
+                        v_reduce(pk1, s1);
+                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                        __builtin_amdgcn_wave_barrier();
 #pragma unroll
                         for (int m = 0; m < L::MPL; ++m)
 #pragma unroll
@@ -1337,7 +1364,7 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
                 }
                 for (; u * L::TPW < vn; u += kNW) {
                     f16x2_t s0[L::MPL][L::HW];
-                    v_pass(u, s0);
+                    v_pass(u, s0, cur, [&]() { if ((u + kNW) * L::TPW < vn) load_pre(u + kNW, cur); });
                     v_flush(s0);
                 }
             }
