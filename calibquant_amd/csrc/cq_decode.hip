@@ -389,7 +389,10 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
             }
         }
     };
-    phase_priority(std::integral_constant<int, 0>{});
+    // (unconditional at entry - with no later change every wave simply runs at this priority - so that no branch
+    // on a kernel argument stands between the wave's start and the loads of the other arguments: all of them are
+    // then requested in one go instead of in two round trips)
+    if constexpr (NT == 512) __builtin_amdgcn_s_setprio(2);
 
     uint32_t vb = static_cast<uint32_t>(virtual_block_id());
     uint32_t qn = g.d_ng.quot(vb);
@@ -456,11 +459,16 @@ __global__ __launch_bounds__(NT, 4) void decode_kernel(DecodeGeom g) {
     constexpr int LPR = L::LPR, NKP = L::NKP, RPW = L::RPW;
     const int lq = tid % LPR, krow = tid / LPR;
     const int wvr = __builtin_amdgcn_readfirstlane(wv);   // wave-uniform: scalar row arithmetic
-    const int64_t res_off = do_res ? b * g.rs_b + hkv * g.rs_h : 0;   // one offset for both windows
+    // (the strides are read where the other kernel arguments are, not behind the branch that needs them: one
+    // round trip to the argument block instead of one more)
+    // (a single launch: every workgroup has a window; of a chunked launch only the residual units do)
+    int64_t arg_rs_b = g.rs_b, arg_rs_h = g.rs_h, arg_rs_r = g.rs_r;
+    if constexpr (!CHUNKED) asm volatile("" : "+s"(arg_rs_b), "+s"(arg_rs_h), "+s"(arg_rs_r));
+    const int64_t res_off = do_res ? b * arg_rs_b + hkv * arg_rs_h : 0;   // one offset for both windows
     const uint16_t* kb = static_cast<const uint16_t*>(do_res ? g.kres : g.q) + res_off;
     const uint16_t* vbp = static_cast<const uint16_t*>(do_res ? g.vres : g.q) + res_off;
     const int last_r = do_res ? R - 1 : 0;
-    const int64_t rs_r = do_res ? g.rs_r : 0;
+    const int64_t rs_r = do_res ? arg_rs_r : 0;
     uint4 rk[NKP];
     uint32_t rv[RPW];
     auto load_res_k = [&](int r0, uint4* k2) {   // rows past R re-read row R-1 (their logit is masked)
