@@ -151,8 +151,9 @@ def test_quantize_pack_full_size_properties(ops, bits):
 # rows per thread); the other shapes take three launches.
 LONG_SHAPES = [(2, 9984, 8, 128),    # 4 x 2496 -> 10: the 26B prompt's token count
                (3, 3329, 2, 128),    # just beyond one workgroup: three launches
-               (1, 13000, 1, 128),   # 4 x 3250 -> 13
-               (1, 40000, 1, 128),   # 16 x 2500 -> 10
+               (4, 13000, 1, 128),   # 4 x 3250 -> 13
+               (2, 40000, 2, 128),   # 16 x 2500 -> 10
+               (1, 40000, 1, 128),   # a single (batch, head) pair: three launches
                (9, 5000, 8, 128),    # 2 x 2500 -> 10; 288 slices x 2 parts: more ids than workgroups, 3 steps
                (2, 7000, 8, 128)]    # three launches
 
